@@ -9,14 +9,14 @@ duplicate ``register_sequence`` raises "already registered" (:150-156).
 
 Beyond the reference: a layer says what it keeps per token (a ``PagedSpec``: the
 tensors of a page, a window, a page size of its own if its kernels want one) and
-layers are put into *groups* by window and page size.  The layers of a group
+layers are put into *groups* by window (with the first tokens it keeps) and page size.  The layers of a group
 share one page pool and one block table per request; each has tensors of its own,
 allocated as its spec lists them.  A group with a window releases a page as soon
-as the window has passed it, while the request is still live.  Every group's pool
+as the window has passed it, while the request is still live, unless the page
+holds some of the request's first tokens that the window keeps visible.  Every group's pool
 holds the same number of tokens, ``num_blocks * block_size``, cut into pages of
 the group's size.  Mixers with fixed-size state get one slot per request in a
-state tensor (this architecture has none; the slot is assigned all the same so
-nothing changes when one is added).
+state tensor, zeroed when the request is registered.
 """
 
 from __future__ import annotations
@@ -38,6 +38,7 @@ class PagedGroup:
     window: int | None
     pool: PagePool
     page_size: int = 0
+    keep_first: int = 0                                  # a request's first tokens that stay beside the window
     runs: list[int] = field(default_factory=list)      # layer runs whose tensors use this group's page ids
 
 
@@ -72,17 +73,18 @@ class CacheManager:
         self.dtype, self.device = dtype, torch.device(device)
         self.groups: list[PagedGroup] = []
         self.layer_caches: list[LayerCache | None] = [None] * len(needs)
-        by_need: dict[tuple[int | None, int], int] = {}
+        by_need: dict[tuple[int | None, int, int], int] = {}
         for run, need in enumerate(needs):
             if isinstance(need, PagedSpec):
                 page_size = int(need.page_size or self.block_size)
-                key = (need.window, page_size)
+                keep_first = int(need.keep_first) if need.window is not None else 0
+                key = (need.window, page_size, keep_first)
                 if key not in by_need:
                     pages = self.pool_tokens // page_size
                     if pages < 1:
                         raise ValueError(f"a pool of {self.pool_tokens} tokens holds no page of {page_size}")
                     by_need[key] = len(self.groups)
-                    self.groups.append(PagedGroup(need.window, PagePool(pages), page_size))
+                    self.groups.append(PagedGroup(need.window, PagePool(pages), page_size, keep_first))
                 group = by_need[key]
                 self.groups[group].runs.append(run)
                 tensors = {}
@@ -231,9 +233,11 @@ class CacheManager:
             if group.window is None:
                 continue
             # The next token sits at position num_tokens and sees keys from
-            # num_tokens - window + 1 on; pages wholly below that are done.
+            # num_tokens - window + 1 on; pages wholly below that are done, but for
+            # the pages that hold any of the request's kept first tokens.
             first_visible = record.num_tokens - group.window + 1
-            for logical in range(min(len(pages), max(0, first_visible) // group.page_size)):
+            kept_pages = self._pages_for(group, group.keep_first)
+            for logical in range(kept_pages, min(len(pages), max(0, first_visible) // group.page_size)):
                 if pages[logical] != RELEASED:
                     group.pool.release(pages[logical])
                     pages[logical] = RELEASED

@@ -129,6 +129,8 @@ def architecture_of(data: dict[str, Any]) -> str:
     folder written by any exporter carries, so it is the registry's key here.
     """
     archs = data.get("architectures")
+    if archs is None and isinstance(data.get("architecture"), str):
+        return data["architecture"]          # a config.json that names its one architecture directly
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
         raise ConfigError("config.json: 'architectures' must be a non-empty list of strings")
     return archs[0]

@@ -140,3 +140,88 @@ extern "C" int somi_rope_kv_store(void* qkv, int dtype, int64_t row_stride, cons
     SOMI_LAUNCH_CHECK("rope_kv_store");
     return 0;
 }
+
+// The general form: key heads and value heads differ in number and size, and the rotation may pair neighbouring
+// channels.  A row holds nq query heads of dk channels, then nk key heads of dk, then nv value heads of dv.  The first
+// 2 * rot_half channels of every query and key head are rotated: channel j with j + rot_half (pairs == 0), or
+// channel 2 j with 2 j + 1 (pairs == 1); the pair (u, w) at position p becomes (u cos a - w sin a, w cos a + u sin a),
+// a = p * inv_freq[j].  The rest pass.  K cache: [pages, nk, page_size, dk]; V cache: [pages, nv, dv, page_size].
+template <typename T>
+__global__ void __launch_bounds__(ROPE_THREADS)
+rope_kv_store_general_kernel(T* __restrict__ qkv, int64_t row_stride, const int* __restrict__ positions,
+                             const int* __restrict__ slots, const float* __restrict__ inv_freq, int rot_half, int pairs,
+                             int nq, int nk, int dk, int nv, int dv, T* __restrict__ kc, T* __restrict__ vc,
+                             int page_size) {
+    __shared__ float cs[2][ROPE_MAX_HALF];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    T* row = qkv + (int64_t)t * row_stride;
+    if (rot_half > 0) {
+        const float pos = (float)positions[t];
+        for (int j = tid; j < rot_half; j += ROPE_THREADS) {
+            const float angle = pos * inv_freq[j];
+            cs[0][j] = cosf(angle);
+            cs[1][j] = sinf(angle);
+        }
+    }
+    __syncthreads();
+    const int slot = (nk > 0 || nv > 0) ? slots[t] : -1;       // -1: a token without a cache slot (padding)
+    const int64_t page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+    // q (in place) and k (into its page): the rotated pairs
+    for (int item = tid; item < (nq + nk) * rot_half; item += ROPE_THREADS) {
+        const int hh = item / rot_half, j = item % rot_half;
+        const int first = pairs ? 2 * j : j, second = pairs ? 2 * j + 1 : j + rot_half;
+        const T* src = row + (int64_t)hh * dk;
+        T* dst = row + (int64_t)hh * dk;
+        if (hh >= nq) {
+            if (slot < 0) continue;
+            dst = kc + ((page * nk + (hh - nq)) * page_size + off) * dk;
+        }
+        const float u = to_float(src[first]), w = to_float(src[second]);
+        const float c = cs[0][j], sn = cs[1][j];
+        dst[first] = from_float<T>(u * c - w * sn);
+        dst[second] = from_float<T>(w * c + u * sn);
+    }
+    // k: the channels past the rotated ones go to the page as they are
+    const int rest = dk - 2 * rot_half;
+    if (slot >= 0 && rest > 0)
+        for (int item = tid; item < nk * rest; item += ROPE_THREADS) {
+            const int hh = item / rest, d = 2 * rot_half + item % rest;
+            kc[((page * nk + hh) * page_size + off) * dk + d] = row[(int64_t)(nq + hh) * dk + d];
+        }
+    // v: into its page, transposed
+    if (slot >= 0)
+        for (int item = tid; item < nv * dv; item += ROPE_THREADS) {
+            const int hh = item / dv, d = item % dv;
+            vc[((page * nv + hh) * (int64_t)dv + d) * page_size + off] = row[(int64_t)(nq + nk) * dk + (int64_t)hh * dv + d];
+        }
+}
+
+// inv_freq: [rotary_dim / 2] float32, or null for no rotation.  With nk == 0 and nv == 0 only q is rotated.
+extern "C" int somi_rope_kv_store_general(void* qkv, int dtype, int64_t row_stride, const int* positions,
+                                          const int* slots, const float* inv_freq, int rotary_dim, int pairs,
+                                          int n_tokens, int nq, int nk, int dk, int nv, int dv, void* k_cache,
+                                          void* v_cache, int page_size, hipStream_t stream) {
+    SOMI_REQUIRE(n_tokens >= 0 && nq >= 0 && nk >= 0 && nv >= 0 && dk > 0 && dv > 0, "rope_kv_store_general: bad sizes");
+    SOMI_REQUIRE(rotary_dim >= 0 && rotary_dim <= dk && rotary_dim % 2 == 0,
+                 "rope_kv_store_general: rotary_dim %d must be even and <= the key size %d", rotary_dim, dk);
+    SOMI_REQUIRE(row_stride >= (int64_t)(nq + nk) * dk + (int64_t)nv * dv, "rope_kv_store_general: row stride %lld too small",
+                 (long long)row_stride);
+    SOMI_REQUIRE((nk == 0 || k_cache) && (nv == 0 || v_cache) && ((nk == 0 && nv == 0) || (slots && page_size > 0)),
+                 "rope_kv_store_general: cache pointers, slots and page size are needed when k/v heads are given");
+    SOMI_REQUIRE(rotary_dim / 2 <= ROPE_MAX_HALF, "rope_kv_store_general: rotary_dim %d is more than %d", rotary_dim,
+                 2 * ROPE_MAX_HALF);
+    if (n_tokens == 0 || nq + nk + nv == 0) return 0;
+    const int rot_half = inv_freq ? rotary_dim / 2 : 0;
+    if (dtype == SOMI_F32)
+        hipLaunchKernelGGL(rope_kv_store_general_kernel<float>, dim3(n_tokens), dim3(ROPE_THREADS), 0, stream,
+                           (float*)qkv, row_stride, positions, slots, inv_freq, rot_half, pairs, nq, nk, dk, nv, dv,
+                           (float*)k_cache, (float*)v_cache, page_size);
+    else if (dtype == SOMI_BF16)
+        hipLaunchKernelGGL(rope_kv_store_general_kernel<bf16>, dim3(n_tokens), dim3(ROPE_THREADS), 0, stream,
+                           (bf16*)qkv, row_stride, positions, slots, inv_freq, rot_half, pairs, nq, nk, dk, nv, dv,
+                           (bf16*)k_cache, (bf16*)v_cache, page_size);
+    else
+        return somi_fail("rope_kv_store_general: unknown dtype %d", dtype);
+    SOMI_LAUNCH_CHECK("rope_kv_store_general");
+    return 0;
+}

@@ -708,3 +708,154 @@ def probe_mfma(iters: int, device: torch.device | str = "cuda:0", dense: bool = 
     flops = ctypes.c_double(0.0)
     _check(library().somi_probe_mfma(int(iters), 1 if dense else 0, _ptr(sink), ctypes.byref(flops), _stream()))
     return float(flops.value)
+
+
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def act_mul(gate_up: torch.Tensor, activation: str) -> torch.Tensor:
+    """act(gate) * up for gate_up = [gate columns | up columns]; ``activation``: one of ACTIVATIONS."""
+    _need(gate_up, "gate_up")
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"act_mul: unknown activation {activation!r}; known: {sorted(ACTIVATIONS)}")
+    n, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelError(f"act_mul: width {two_i} is odd")
+    out = torch.empty((n, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _check(library().somi_act_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), n, two_i // 2,
+                                  ACTIVATIONS[activation], _stream()))
+    return out
+
+
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap * tanh(x / cap), in place on float32 values."""
+    _need(x, "logits", torch.float32)
+    _check(library().somi_softcap(_ptr(x), ctypes.c_float(cap), ctypes.c_int64(x.numel()), _stream()))
+    return x
+
+
+def rope_kv_store_general(qkv: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
+                          inv_freq: torch.Tensor | None, rotary_dim: int, pairs: bool, nq: int, nk: int, dk: int,
+                          nv: int, dv: int, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None) -> None:
+    """Rotate the nq query heads (in place) and the nk key heads of size dk of every row of ``qkv`` ([N, >= (nq + nk) dk
+    + nv dv]: queries, keys, values side by side) and store keys and values in their pages.  ``pairs``: the rotation
+    pairs channel 2j with 2j + 1 instead of j with j + rotary_dim / 2.  k cache: [pages, nk, page, dk]; v cache:
+    [pages, nv, dv, page]; nk == nv == 0 rotates the queries only."""
+    _need(qkv, "qkv")
+    n = qkv.shape[0]
+    if qkv.shape[1] < (nq + nk) * dk + nv * dv:
+        raise KernelError(f"rope_kv_store_general: rows of {qkv.shape[1]} are narrower than {(nq + nk) * dk + nv * dv}")
+    _need(positions, "positions", torch.int32, (n,))
+    page_size = 0
+    if nk or nv:
+        _need(slots, "slot mapping", torch.int32, (n,))
+        _need(k_cache, "k cache", qkv.dtype)
+        _need(v_cache, "v cache", qkv.dtype)
+        if k_cache.dim() != 4 or k_cache.shape[1] != nk or k_cache.shape[3] != dk:
+            raise KernelError(f"rope_kv_store_general: k cache {tuple(k_cache.shape)} != [pages, {nk}, page, {dk}]")
+        page_size = k_cache.shape[2]
+        if tuple(v_cache.shape) != (k_cache.shape[0], nv, dv, page_size):
+            raise KernelError(f"rope_kv_store_general: v cache {tuple(v_cache.shape)} != "
+                              f"[{k_cache.shape[0]}, {nv}, {dv}, {page_size}]")
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", torch.float32, (rotary_dim // 2,))
+    _check(library().somi_rope_kv_store_general(
+        _ptr(qkv), dtype_code(qkv.dtype), ctypes.c_int64(qkv.shape[1]), _ptr(positions), _ptr(slots), _ptr(inv_freq),
+        int(rotary_dim), 1 if pairs else 0, n, nq, nk, dk, nv, dv, _ptr(k_cache if nk else None),
+        _ptr(v_cache if nv else None), page_size, _stream()))
+
+
+def diff_attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                         token_entry: torch.Tensor, positions: torch.Tensor, nq: int, window: int, keep_first: int,
+                         scale: float, lam: float, eps: float, out_scale: float,
+                         out: torch.Tensor | None = None, token_list: torch.Tensor | None = None) -> torch.Tensor:
+    """Differential attention of the listed tokens (all when ``token_list`` is None) over their requests' pages with the
+    plain float32 kernel: per head two softmax maps over the same values, a1 - lam * a2, divided by its root mean
+    square over the head's value channels, times ``out_scale`` -> [N, nq * dv].  q: row t holds token t's 2 nq
+    query maps of dk channels first; k cache: [pages, 2 nkv, page, dk]; v cache: [pages, nkv, dv, page].  A token
+    sees the keys within ``window`` positions (0: all) and the first ``keep_first`` of its request."""
+    _need(q, "q")
+    n = q.shape[0]
+    _need(k_cache, "k cache", q.dtype)
+    _need(v_cache, "v cache", q.dtype)
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.shape[1] != 2 * v_cache.shape[1]:
+        raise KernelError("diff_attention: caches must be k [pages, 2 kv_heads, page, dk] and v [pages, kv_heads, dv, page]")
+    pages, nkv, dv, page_size = v_cache.shape
+    dk = k_cache.shape[3]
+    if k_cache.shape[0] != pages or k_cache.shape[2] != page_size:
+        raise KernelError(f"diff_attention: k cache {tuple(k_cache.shape)} and v cache {tuple(v_cache.shape)} disagree")
+    if q.shape[1] < 2 * nq * dk:
+        raise KernelError("diff_attention: q rows are narrower than 2 * heads * dk")
+    _need(block_table, "block table", torch.int32)
+    _need(token_entry, "token entries", torch.int32, (n,))
+    _need(positions, "positions", torch.int32, (n,))
+    if out is None:
+        out = torch.empty((n, nq * dv), dtype=q.dtype, device=q.device)
+    _need(out, "attention out", q.dtype, (n, nq * dv))
+    n_list = n
+    if token_list is not None:
+        _need(token_list, "token list", torch.int32)
+        n_list = token_list.numel()
+    _check(library().somi_diff_attention_plain(
+        _ptr(q), dtype_code(q.dtype), ctypes.c_int64(q.shape[1]), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
+        block_table.shape[1], _ptr(token_list), _ptr(token_entry), _ptr(positions), n_list, nq, nkv, dk, dv, page_size,
+        int(window), int(keep_first), ctypes.c_float(scale), ctypes.c_float(lam), ctypes.c_float(eps),
+        ctypes.c_float(out_scale), _ptr(out), _stream()))
+    return out
+
+
+def gla_decay(a: torch.Tensor, w2: torch.Tensor, bias: torch.Tensor | None, tau: float) -> torch.Tensor:
+    """alpha = sigmoid(a @ w2.T + bias)^(1 / tau) in float32 -> [N, channels].  a: [N, rank] (a view with a row stride of
+    its own is taken as it is); w2: [channels, rank]."""
+    if not isinstance(a, torch.Tensor) or not a.is_cuda or a.dim() != 2 or a.stride(1) != 1:
+        raise KernelError("gla_decay: the input must be a matrix on the GPU with contiguous rows")
+    n, rank = a.shape
+    _need(w2, "decay weight", a.dtype)
+    if w2.dim() != 2 or w2.shape[1] != rank:
+        raise KernelError(f"gla_decay: weight {tuple(w2.shape)} does not fit a rank of {rank}")
+    channels = w2.shape[0]
+    if bias is not None:
+        _need(bias, "decay bias", torch.float32, (channels,))
+    alpha = torch.empty((n, channels), dtype=torch.float32, device=a.device)
+    _check(library().somi_gla_decay(_ptr(a), dtype_code(a.dtype), ctypes.c_int64(a.stride(0)), _ptr(w2), _ptr(bias),
+                                    ctypes.c_float(tau), _ptr(alpha), n, channels, rank, _stream()))
+    return alpha
+
+
+def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, alpha: torch.Tensor, entry_start: torch.Tensor,
+             state_slots: torch.Tensor, state: torch.Tensor, q_scale: float) -> torch.Tensor:
+    """The recurrence S <- diag(alpha_t) S + k_t v_t^T, o_t = S^T (q_t * q_scale) per head over the tokens of every entry,
+    from and into ``state[state_slots[e]]`` ([slots, heads, dim, vdim] float32) -> o [N, heads, vdim] float32.
+    q, k: [N, heads * dim] and v: [N, heads * vdim], views of one matrix (one row stride)."""
+    slots, heads, dim, vdim = state.shape
+    _need(state, "recurrent state", torch.float32)
+    n = q.shape[0]
+    for t, name, width in ((q, "q", heads * dim), (k, "k", heads * dim), (v, "v", heads * vdim)):
+        if (not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != q.dtype or t.dim() != 2 or t.stride(1) != 1
+                or t.stride(0) != q.stride(0) or tuple(t.shape) != (n, width)):
+            raise KernelError(f"gla_scan: {name} must be [{n}, {width}] of {q.dtype} with the row stride of q")
+    _need(alpha, "decays", torch.float32, (n, heads * dim))
+    entries = state_slots.numel()
+    _need(entry_start, "entry offsets", torch.int32, (entries + 1,))
+    _need(state_slots, "state slots", torch.int32, (entries,))
+    o = torch.empty((n, heads, vdim), dtype=torch.float32, device=q.device)
+    _check(library().somi_gla_scan(_ptr(q), _ptr(k), _ptr(v), dtype_code(q.dtype), ctypes.c_int64(q.stride(0)),
+                                   _ptr(alpha), _ptr(entry_start), _ptr(state_slots), _ptr(state), entries, heads, dim,
+                                   vdim, ctypes.c_float(q_scale), _ptr(o), _stream()))
+    return o
+
+
+def gla_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, eps: float) -> torch.Tensor:
+    """o / sqrt(mean(o^2) + eps) * weight * silu(gate) per head -> [N, heads * vdim] in the gate's dtype.  o: [N, heads,
+    vdim] float32; weight: [vdim] float32; gate: [N, heads * vdim] (a view with a row stride of its own is fine)."""
+    _need(o, "recurrence output", torch.float32)
+    n, heads, vdim = o.shape
+    _need(weight, "norm weight", torch.float32, (vdim,))
+    if (not isinstance(gate, torch.Tensor) or not gate.is_cuda or gate.dim() != 2 or gate.stride(1) != 1
+            or tuple(gate.shape) != (n, heads * vdim)):
+        raise KernelError(f"gla_norm_gate: the gate must be [{n}, {heads * vdim}] on the GPU with contiguous rows")
+    y = torch.empty((n, heads * vdim), dtype=gate.dtype, device=o.device)
+    _check(library().somi_gla_norm_gate(_ptr(o), _ptr(weight), _ptr(gate), dtype_code(gate.dtype),
+                                        ctypes.c_int64(gate.stride(0)), ctypes.c_float(eps), _ptr(y), n, heads, vdim,
+                                        _stream()))
+    return y

@@ -51,6 +51,8 @@ class GroupedQueryAttention(Mixer):
         self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
         self.shares_cache = bool(shares_cache)     # reads the cache another layer writes: no k/v of its own
         self.position = build_part("position", position, prefix=self.name(self.names["position"]))
+        if getattr(self.position, "pairing", "half") != "half":
+            raise ValueError(f"{prefix}: this part's kernels rotate channel j with j + rotary_dim / 2 only")
 
     ROLES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "position": "rotary_emb"}
 

@@ -85,13 +85,15 @@ class PageTensor:
 @dataclass(frozen=True)
 class PagedSpec:
     """Something kept for every past token, in pages: the tensors a page holds, how many of the latest tokens
-    stay visible (``window``, the current one included; None = all), and the page size the mixer's kernels want
-    (None = the engine's).  Layers whose window and page size agree share one pool of pages and one block table
-    per request; each layer run has its own tensors."""
+    stay visible (``window``, the current one included; None = all), how many of a request's first tokens stay
+    visible beside the window (``keep_first``), and the page size the mixer's kernels want (None = the engine's).
+    Layers whose window, kept tokens and page size agree share one pool of pages and one block table per request;
+    each layer run has its own tensors."""
 
     tensors: tuple[PageTensor, ...]
     window: int | None = None
     page_size: int | None = None
+    keep_first: int = 0
 
     def __post_init__(self) -> None:
         names = [t.name for t in self.tensors]
@@ -99,6 +101,8 @@ class PagedSpec:
             raise ValueError(f"a paged cache needs at least one tensor and distinct names, got {names}")
         if self.page_size is not None and self.page_size < 1:
             raise ValueError(f"page size {self.page_size} must be >= 1")
+        if self.keep_first < 0 or (self.window is not None and self.window < 1):
+            raise ValueError(f"a window must be >= 1 and kept tokens >= 0, got {self.window} and {self.keep_first}")
 
 
 class PagedKVSpec(PagedSpec):
@@ -163,6 +167,9 @@ class Part:
         self.prefix = prefix
 
     def name(self, suffix: str) -> str:
+        """``prefix.suffix``; an empty prefix or suffix leaves the other alone."""
+        if not suffix:
+            return self.prefix
         return f"{self.prefix}.{suffix}" if self.prefix else suffix
 
     def weight_specs(self) -> list[WeightSpec]:

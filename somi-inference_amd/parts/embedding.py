@@ -19,17 +19,19 @@ from .base import Fetch, Part, Runtime
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, prefix: str, vocab_size: int, hidden_size: int) -> None:
+    def __init__(self, prefix: str, vocab_size: int, hidden_size: int, tensor: str = "weight") -> None:
+        """``tensor``: what the checkpoint calls the table under the part's prefix."""
         super().__init__(prefix)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.tensor = str(tensor)
         self.weight: torch.Tensor | None = None
 
     def weight_specs(self) -> list[WeightSpec]:
-        return [WeightSpec(self.name("weight"), (self.vocab_size, self.hidden_size), MATRIX)]
+        return [WeightSpec(self.name(self.tensor), (self.vocab_size, self.hidden_size), MATRIX)]
 
     def load(self, fetch: Fetch, runtime: Runtime) -> None:
         super().load(fetch, runtime)
-        self.weight = fetch(self.name("weight"))
+        self.weight = fetch(self.name(self.tensor))
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         """[N] int32 -> [N, H] float32 (the residual stream starts in float32)."""
@@ -37,23 +39,29 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
-    """logits = x . W^T in float32, for the rows that were asked for only."""
+    """logits = x . W^T in float32, for the rows that were asked for only; with ``softcap`` c the logits are then
+    bounded smoothly, c * tanh(logits / c)."""
     graph_safe = True
 
-    def __init__(self, prefix: str, vocab_size: int, hidden_size: int, tied: bool = False) -> None:
+    def __init__(self, prefix: str, vocab_size: int, hidden_size: int, tied: bool = False,
+                 softcap: float | None = None, tensor: str = "weight") -> None:
         super().__init__(prefix)
         self.vocab_size, self.hidden_size, self.tied = int(vocab_size), int(hidden_size), bool(tied)
+        self.softcap = float(softcap) if softcap else None
+        if self.softcap is not None and not self.softcap > 0.0:
+            raise ValueError(f"{prefix}: a soft cap must be > 0, got {softcap}")
+        self.tensor = str(tensor)
         self.weight: torch.Tensor | None = None
 
     def weight_specs(self) -> list[WeightSpec]:
         if self.tied:
             return []
-        return [WeightSpec(self.name("weight"), (self.vocab_size, self.hidden_size), MATRIX)]
+        return [WeightSpec(self.name(self.tensor), (self.vocab_size, self.hidden_size), MATRIX)]
 
     def load(self, fetch: Fetch, runtime: Runtime) -> None:
         super().load(fetch, runtime)
         if not self.tied:
-            self.weight = fetch(self.name("weight"))
+            self.weight = fetch(self.name(self.tensor))
 
     def tie(self, embedding: TokenEmbedding) -> None:
         self.weight = embedding.weight
@@ -63,4 +71,7 @@ class LMHead(Part):
         return 2.0 * tokens * self.vocab_size * self.hidden_size
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return linear_kernels.linear(x, self.weight, None, torch.float32)
+        logits = linear_kernels.linear(x, self.weight, None, torch.float32)
+        if self.softcap is not None:
+            ops.softcap_(logits, self.softcap)
+        return logits

@@ -16,19 +16,21 @@ class RMSNorm(Norm):
     fusable = True        # weight * (h / sqrt(mean(h^2) + eps)): what a projection can apply while it loads h
 
     def __init__(self, prefix: str, hidden_size: int, eps: float,
-                 init: tuple[float, float] = (1.0, 0.1)) -> None:
+                 init: tuple[float, float] = (1.0, 0.1), tensor: str = "weight") -> None:
+        """``tensor``: what the checkpoint calls the scale under the part's prefix."""
         super().__init__(prefix)
+        self.tensor = str(tensor)
         self.hidden_size = int(hidden_size)
         self.eps = float(eps)
         self._init = Init(*init)
         self.weight: torch.Tensor | None = None
 
     def weight_specs(self) -> list[WeightSpec]:
-        return [WeightSpec(self.name("weight"), (self.hidden_size,), VECTOR, self._init)]
+        return [WeightSpec(self.name(self.tensor), (self.hidden_size,), VECTOR, self._init)]
 
     def load(self, fetch: Fetch, runtime: Runtime) -> None:
         super().load(fetch, runtime)
-        self.weight = fetch(self.name("weight"))
+        self.weight = fetch(self.name(self.tensor))
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return ops.rmsnorm(h, self.weight, self.eps, self.runtime.dtype)

@@ -29,7 +29,7 @@ from ..engine.batch import StepEntry
 from ..models.loader import load_model, make_runner, random_model
 
 DEFAULT_PAGE_TOKENS = 16      # tokens per cache page unless asked otherwise; divides the 64 that --max-tokens is counted in
-DEFAULT_MAX_REQUESTS = 64     # request slots of the cache manager (a trace holds a handful live)
+DEFAULT_MAX_REQUESTS = 4      # request slots of the cache manager: a trace holds at most four live, so slots are used again
 RANDOM_PREFIX = "random:"
 
 

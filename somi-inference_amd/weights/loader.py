@@ -62,7 +62,7 @@ def check_weights(specs: Iterable[WeightSpec], source: WeightSource,
     for name, spec in wanted.items():
         if name not in present:
             continue
-        if tuple(source.shape(name)) != spec.shape:
+        if not spec.fits(source.shape(name)):
             wrong_shape.append((name, tuple(source.shape(name)), spec.shape))
         stored = source.stored_dtype(name)
         if spec.role == TABLE and stored.is_floating_point:

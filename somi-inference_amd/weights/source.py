@@ -85,6 +85,9 @@ def random_tensor(spec: WeightSpec, seed: int, device: torch.device | str,
     written on the CPU and tensors made on the GPU from the same seed are
     different (equally valid) models.
     """
+    if spec.open_sizes:
+        raise ValueError(f"tensor {spec.name!r} leaves a size to the checkpoint ({spec.shape}): random weights need "
+                         f"the configuration to give it")
     device = torch.device(device)
     gen = torch.Generator(device=device)
     gen.manual_seed(tensor_seed(seed, spec.name))

@@ -7,6 +7,7 @@ from dataclasses import dataclass
 MATRIX = "matrix"   # operand of a matrix product: held in the engine's compute dtype
 VECTOR = "vector"   # norm scale or bias: held in float32 (a 32-bit stored tensor stays 32-bit)
 TABLE = "table"     # integer table: held as int32
+ANY_SIZE = -1       # in a declared shape: a size that the checkpoint's tensor gives
 
 
 @dataclass(frozen=True)
@@ -28,3 +29,13 @@ class WeightSpec:
         if self.role not in (MATRIX, VECTOR, TABLE):
             raise ValueError(f"weight {self.name!r}: unknown role {self.role!r}")
         object.__setattr__(self, "shape", tuple(int(s) for s in self.shape))
+
+    def fits(self, shape) -> bool:
+        """Whether a stored tensor of ``shape`` is what the part declared; a declared size of ANY_SIZE is one that
+        the checkpoint gives (the part reads it from the tensor)."""
+        shape = tuple(int(s) for s in shape)
+        return len(shape) == len(self.shape) and all(want in (ANY_SIZE, got) for want, got in zip(self.shape, shape))
+
+    @property
+    def open_sizes(self) -> bool:
+        return ANY_SIZE in self.shape
