@@ -154,8 +154,15 @@ class ModelRunner:
         if device_tokens is not None:
             static.batch.token_ids[:len(entries)].copy_(device_tokens)
         # once outside a capture: lazy initialisation (library handles, first allocations) must
-        # not happen while the stream is being recorded; the step's writes are simply redone
+        # not happen while the stream is being recorded.  What the step writes into pages is simply
+        # written again by the replay; recurrent state that the step advances is put back first.
+        stateful = [cache for cache in self.cache.layer_caches
+                    if cache is not None and cache.state is not None and cache.writes]
+        slots = static.batch.state_slots.to(torch.int64) if stateful else None
+        before = [cache.state.index_select(0, slots) for cache in stateful]
         self.model.forward(static.batch, self.cache.layer_caches)
+        for cache, rows in zip(stateful, before):
+            cache.state.index_copy_(0, slots, rows)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
