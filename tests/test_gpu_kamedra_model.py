@@ -1,0 +1,188 @@
+"""The Kamedra decoder in the engine against the plain implementation, for every way of cutting the work."""
+
+import pytest
+import torch
+
+import helpers
+from helpers import make_engine, mixed_trace, peak_pages, run_portions, token_ids
+from kamedra_helpers import KAMEDRA, load_plain, write_kamedra
+from plain import kamedra_plain as plain
+from somi_inference_amd.engine import StepEntry
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+
+# The float32 engine against the float32 plain implementation: sums in another order only, but this design divides
+# every head's output by its own root mean square, which passes rounding on more strongly than a softmax does.
+KAMEDRA_F32_TOL = dict(atol=1e-4, rtol=2e-4)
+
+
+# bfloat16: the shares of the other architecture's tests for a tensor (root mean square error 3 % of the logits', no
+# element off by more than 5 % of the largest logit); a single row may be off by 10 % of its own size instead of 6 %
+# (correct runs of these models measure up to 7.4 %; a row computed from a wrong key, state or page is off by its own size).
+KAMEDRA_ROW_RMS_SHARE = 0.10
+
+
+def assert_close(got, want, dtype, what="", per_row=False):
+    if dtype == "float32":
+        torch.testing.assert_close(got.float().cpu(), want.float().cpu(), msg=lambda m: f"{what}: {m}", **KAMEDRA_F32_TOL)
+        return
+    helpers.assert_close(got, want, dtype, what, per_row=False)
+    if per_row:
+        error, want = (got.float().cpu() - want.float().cpu()), want.float().cpu()
+        share = error.pow(2).mean(dim=-1).sqrt() / want.pow(2).mean(dim=-1).sqrt()
+        over = (share > KAMEDRA_ROW_RMS_SHARE).nonzero().flatten().tolist()
+        assert not over, f"{what}: rows {over[:8]} are off by {[round(float(share[i]), 4) for i in over[:8]]} of their own size"
+NAMES = list(KAMEDRA)
+KINDS = {"plain": (1.0, False), "peaky": (2.0, True)}      # (scale of attention scores, recurrent layers made steady)
+
+
+def skip_unsteady_bfloat16(kind, dtype):
+    if dtype == "bfloat16" and not KINDS[kind][1]:
+        pytest.skip("bfloat16 is held to a bound on models whose recurrent heads are steady at the first tokens")
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("kamedra")
+    return {(kind, name): write_kamedra(name, str(root / f"{kind}_{name}"), peaky, steady)
+            for kind, (peaky, steady) in KINDS.items() for name in NAMES}
+
+
+@pytest.fixture(scope="module")
+def oracle(folders):
+    """Plain logits of (kind, name, tokens), computed once."""
+    cache, models = {}, {}
+
+    def get(kind, name, tokens):
+        key = (kind, name, tuple(tokens))
+        if key not in cache:
+            if (kind, name) not in models:
+                models[(kind, name)] = load_plain(folders[(kind, name)])
+            config, weights = models[(kind, name)]
+            cache[key] = plain.forward(config, weights, list(tokens))
+        return cache[key]
+    return get
+
+
+def vocab_of(name):
+    return KAMEDRA[name]["config"].vocab
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("kind", list(KINDS))
+def test_whole_prompts(kind, name, dtype, folders, oracle):
+    skip_unsteady_bfloat16(kind, dtype)
+    runner, _ = make_engine(folders[(kind, name)], dtype, KAMEDRA[name]["block_size"], 48, max_requests=2)
+    for length, seed in ((1, 1), (2, 2), (9, 3), (33, 4), (64, 5), (131, 6), (300, 7)):
+        tokens = token_ids(vocab_of(name), length, seed)
+        got = run_portions(runner, f"r{length}", tokens, [length])
+        assert_close(got, oracle(kind, name, tokens), dtype, f"{name} {kind} {dtype} whole prompt of {length}", per_row=True)
+    runner.cache.check_invariants()
+    assert runner.cache.free_pages() == [48] * len(runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_prompt_then_long_decoding_token_by_token(name, dtype, folders, oracle):
+    """The decoded tokens pass every window, kept-token and page edge of the configuration."""
+    runner, _ = make_engine(folders[("peaky", name)], dtype, KAMEDRA[name]["block_size"], 24, max_requests=2)
+    for prefill, decoded in ((3, 90), (40, 120)):
+        tokens = token_ids(vocab_of(name), prefill + decoded, 11 * prefill)
+        got = run_portions(runner, "d", tokens, [prefill] + [1] * decoded)
+        assert_close(got, oracle("peaky", name, tokens), dtype, f"{name} {dtype} {prefill} + {decoded} decoded", per_row=True)
+        if dtype == "float32":
+            whole = run_portions(runner, "w", tokens, [prefill + decoded])
+            assert torch.equal(got, whole), "float32 logits differ between decoding and the whole prompt"
+    assert runner.graph_replays > 0          # decoded tokens took the captured step
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_portions_of_several_sizes_down_to_two(name, dtype, folders, oracle):
+    runner, _ = make_engine(folders[("peaky", name)], dtype, KAMEDRA[name]["block_size"], 24, max_requests=2)
+    tokens = token_ids(vocab_of(name), 170, 21)
+    want = oracle("peaky", name, tokens)
+    whole = run_portions(runner, "w", tokens, [170])
+    for sizes in ([2], [7, 2, 5, 3, 11], [16], [17, 15], [64, 2, 1, 1, 40], [1]):
+        got = run_portions(runner, "p", tokens, sizes)
+        assert_close(got, want, dtype, f"{name} {dtype} portions of {sizes}", per_row=True)
+        if dtype == "float32":
+            assert torch.equal(got, whole), f"float32 logits depend on the portions {sizes}"
+    runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_unequal_requests_together_with_pages_and_slots_used_again(name, dtype, folders, oracle):
+    """Up to four live requests (the slots there are), portions beside single tokens, in a pool that only holds what is
+    live: every request's logits equal those it gets alone."""
+    block = KAMEDRA[name]["block_size"]
+    lengths = {"a": 95, "b": 1, "c": 33, "d": 140, "e": 2, "f": 64, "g": 77, "h": 18, "i": 120}
+    requests = {rid: token_ids(vocab_of(name), n, 100 + n) for rid, n in lengths.items()}
+    steps = mixed_trace(requests, seed=5, max_live=4)
+    runner, _ = make_engine(folders[("peaky", name)], dtype, block, peak_pages(steps, block), max_requests=4)
+    alone = {rid: run_portions(runner, "alone", tokens, [len(tokens)]) for rid, tokens in requests.items()}
+    got = {rid: [] for rid in requests}
+    slots_seen = set()
+    for entries, ends in steps:
+        batch = []
+        for rid, start, count in entries:
+            if not runner.cache.has(rid):
+                runner.begin(rid)
+                slots_seen.add(runner.cache.state_slot(rid))
+            batch.append(StepEntry(rid, requests[rid][start:start + count], list(range(count))))
+        logits = runner.step(batch).cpu()
+        at = 0
+        for rid, _, count in entries:
+            got[rid].append(logits[at:at + count].clone())
+            at += count
+        for rid in ends:
+            runner.end(rid)
+        runner.cache.check_invariants()
+    assert len(slots_seen) <= 4 < len(requests)               # slots were used again
+    for rid, tokens in requests.items():
+        rows = torch.cat(got[rid])
+        assert_close(rows, oracle("peaky", name, tokens), dtype, f"{name} {dtype} request {rid} in mixed batches", per_row=True)
+        if dtype == "float32":
+            assert torch.equal(rows, alone[rid]), f"float32 logits of request {rid} depend on the batch"
+    assert runner.cache.free_pages() == [g.pool.num_pages for g in runner.cache.groups]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_slot_used_again_starts_from_zero(dtype, folders):
+    runner, _ = make_engine(folders[("peaky", "A")], dtype, 16, 16, max_requests=1)
+    tokens = token_ids(vocab_of("A"), 40, 9)
+    first = run_portions(runner, "one", tokens, [40])
+    run_portions(runner, "other", token_ids(vocab_of("A"), 55, 10), [30, 25])
+    again = run_portions(runner, "one", tokens, [13, 27])
+    if dtype == "float32":
+        assert torch.equal(first, again)
+    else:
+        assert_close(again, first, dtype, "the same request in a slot that was used in between")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_greedy_generation_through_the_entry_point(name, dtype, folders):
+    from somi_inference_amd import LLM
+    config, weights = load_plain(folders[("peaky", name)])
+    prompts = [token_ids(vocab_of(name), n, 60 + n) for n in (5, 23, 1, 48)]
+    new_tokens = 12
+    llm = LLM(folders[("peaky", name)], dtype=dtype, num_blocks=32, block_size=KAMEDRA[name]["block_size"],
+              max_concurrent=3, max_num_batched_tokens=32, eos_token_id=-1)
+    got = llm.generate(prompts, max_new_tokens=new_tokens, temperature=0.0)
+    for prompt, tokens in zip(prompts, got):
+        assert len(tokens) == new_tokens
+        sequence = list(prompt)
+        for token in tokens:
+            logits = plain.forward(config, weights, sequence)[-1]
+            best = int(logits.argmax())
+            if token != best:
+                # a near tie may flip in bfloat16 (and, by a hair, in another order of float32 sums)
+                gap = float(logits[best] - logits[token])
+                assert gap < (1e-4 if dtype == "float32" else 0.05), f"token {token} instead of {best} (gap {gap})"
+            sequence.append(token)
+    llm.runner.cache.check_invariants()

@@ -1,0 +1,227 @@
+"""Each mechanism of the Kamedra decoder alone: its kernels against the plain functions written from the equations."""
+
+import math
+
+import pytest
+import torch
+
+from plain import kamedra_plain as plain
+from somi_inference_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+def rounded(x: torch.Tensor, dtype) -> torch.Tensor:
+    """float32 values that the dtype holds exactly, so that the kernel and the plain function start from the same."""
+    return x.to(dtype).to(torch.float32)
+
+
+# ------------------------------------------------------------------------------------------ rotation, page store
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nk,dk,nv,dv,dims,page", [(8, 4, 16, 2, 32, 8, 16), (12, 12, 24, 6, 40, 24, 8),
+                                                      (4, 2, 8, 1, 16, 4, 4), (6, 0, 10, 0, 12, 6, 8)])
+def test_pair_rotation_and_page_store(dtype, nq, nk, dk, nv, dv, dims, page):
+    torch.manual_seed(1)
+    n, pages = 37, 12
+    width = (nq + nk) * dk + nv * dv
+    rows = rounded(torch.randn(n, width), dtype)
+    positions = torch.randint(0, 5000, (n,), dtype=torch.int32)
+    slots = torch.randperm(pages * page)[:n].to(torch.int32)
+    slots[5] = -1                                            # a token that stores nothing
+    freqs = plain.rotary_frequencies(dims, 20000.0, dict(factor=8.0, low=1.0, high=4.0, original=2048))
+    qkv = rows.to(dtype).cuda()
+    kc = torch.zeros((pages, max(nk, 1), page, dk), dtype=dtype, device="cuda") if nk else None
+    vc = torch.zeros((pages, max(nv, 1), dv, page), dtype=dtype, device="cuda") if nv else None
+    ops.rope_kv_store_general(qkv, positions.cuda(), slots.cuda() if nk or nv else None, freqs.cuda(), dims, True,
+                              nq, nk, dk, nv, dv, kc, vc)
+    heads = rows[:, :(nq + nk) * dk].view(n, nq + nk, dk)
+    want = plain.rotate_pairs(heads, positions, freqs)
+    torch.testing.assert_close(qkv[:, :nq * dk].float().cpu().view(n, nq, dk), want[:, :nq], **tol(dtype))
+    for t in range(n):
+        slot = int(slots[t])
+        if slot < 0 or not nk:
+            continue
+        torch.testing.assert_close(kc[slot // page, :, slot % page].float().cpu(), want[t, nq:], **tol(dtype))
+        torch.testing.assert_close(vc[slot // page, :, :, slot % page].float().cpu(),
+                                   rows[t, (nq + nk) * dk:].view(nv, dv), **tol(dtype))
+    if nk:
+        assert float(kc.float().abs().sum(dim=(1, 3)).flatten()[torch.tensor(
+            [s for s in range(pages * page) if s not in set(slots.tolist())])].max()) == 0.0   # nothing written elsewhere
+
+
+# ------------------------------------------------------------------------------------------ differential attention
+def paged(keys: torch.Tensor, values: torch.Tensor, page: int, dtype, seed: int):
+    """Pages in shuffled order for keys [T, 2G, dk] and values [T, G, dv] of one request: (k cache, v cache, table)."""
+    t = keys.shape[0]
+    count = (t + page - 1) // page
+    order = torch.randperm(count + 3, generator=torch.Generator().manual_seed(seed))[:count]
+    kc = torch.zeros((count + 3, keys.shape[1], page, keys.shape[2]), dtype=torch.float32)
+    vc = torch.zeros((count + 3, values.shape[1], values.shape[2], page), dtype=torch.float32)
+    for pos in range(t):
+        kc[order[pos // page], :, pos % page] = keys[pos]
+        vc[order[pos // page], :, :, pos % page] = values[pos]
+    return kc.to(dtype).cuda(), vc.to(dtype).cuda(), order.to(torch.int32).view(1, -1).cuda()
+
+
+def plain_differential(q, k, v, heads, scale, size, keep, lam, eps, out_scale):
+    """q: [T, 2H, dk], k: [T, 2G, dk], v: [T, G, dv] -> [T, H * dv] by the plain functions."""
+    g = v.shape[1]
+    out = []
+    for head in range(heads):
+        kv = head // (heads // g)
+        a1 = plain.masked_softmax_attention(q[:, 2 * head], k[:, 2 * kv], v[:, kv], scale, size, keep)
+        a2 = plain.masked_softmax_attention(q[:, 2 * head + 1], k[:, 2 * kv + 1], v[:, kv], scale, size, keep)
+        out.append(plain.rms(a1 - lam * a2, eps) * out_scale)
+    return torch.cat(out, dim=1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,g,dk,dv,page,t,size,keep", [
+    (4, 2, 16, 32, 16, 150, 24, 5), (6, 6, 24, 40, 8, 70, 1000, 0), (2, 1, 8, 16, 4, 90, 7, 9),
+    (3, 1, 48, 32, 16, 300, 130, 17), (2, 2, 20, 130, 8, 40, 1, 0), (4, 4, 32, 16, 32, 260, 128, 128)])
+def test_differential_attention_against_the_plain_maps(dtype, heads, g, dk, dv, page, t, size, keep):
+    torch.manual_seed(2)
+    q = rounded(torch.randn(t, 2 * heads, dk), dtype)
+    k = rounded(torch.randn(t, 2 * g, dk), dtype)
+    v = rounded(torch.randn(t, g, dv), dtype)
+    kc, vc, table = paged(k, v, page, dtype, seed=t)
+    scale, lam, eps, out_scale = 0.4, 0.55, 1e-5, 0.7
+    want = plain_differential(q, k, v, heads, scale, size, keep, lam, eps, out_scale)
+    positions = torch.arange(t, dtype=torch.int32).cuda()
+    entry = torch.zeros(t, dtype=torch.int32).cuda()
+    got = ops.diff_attention_plain(q.view(t, -1).to(dtype).cuda(), kc, vc, table, entry, positions, heads,
+                                   size, keep, scale, lam, eps, out_scale)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype))
+    # a few tokens alone, in another order: the same rows
+    some = torch.tensor([t - 1, 0, t // 2, min(t - 1, keep), min(t - 1, size)], dtype=torch.int32).cuda()
+    out = torch.zeros_like(got)
+    ops.diff_attention_plain(q.view(t, -1).to(dtype).cuda(), kc, vc, table, entry, positions, heads, size, keep, scale,
+                             lam, eps, out_scale, out=out, token_list=some)
+    assert torch.equal(out[some.long()], got[some.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page,size,keep", [(16, 40, 6), (8, 33, 16), (4, 9, 2), (16, 16, 16)])
+def test_one_key_stands_out_exactly_where_the_mask_lets_it(dtype, page, size, keep):
+    """One key carries a large score against every query: a query's output is that key's value (normed) if and only
+    if the key is the query itself, within the window or among the kept first tokens."""
+    torch.manual_seed(3)
+    t, dk, dv = 200, 16, 32
+    direction = torch.nn.functional.normalize(torch.randn(dk), dim=0)
+    for marked in (0, keep - 1, keep, keep + 1, page - 1, page, 3 * page, 77, t - 1):
+        q = rounded(torch.randn(t, 2, dk) * 0.1 + 6.0 * direction, dtype)
+        k = rounded(torch.randn(t, 2, dk) * 0.1, dtype)
+        k[marked] = rounded(6.0 * direction, dtype)
+        v = rounded(torch.randn(t, 1, dv), dtype)
+        kc, vc, table = paged(k, v, page, dtype, seed=marked)
+        got = ops.diff_attention_plain(q.view(t, -1).to(dtype).cuda(), kc, vc, table,
+                                       torch.zeros(t, dtype=torch.int32).cuda(), torch.arange(t, dtype=torch.int32).cuda(),
+                                       1, size, keep, 1.0, 0.0, 1e-6, 1.0).float().cpu()
+        marked_value = plain.rms(v[marked, 0], 1e-6)
+        for i in range(t):
+            sees = plain.visible(i, marked, size, keep)
+            cosine = float(torch.nn.functional.cosine_similarity(got[i], marked_value, dim=0))
+            assert (cosine > 0.999) == sees, f"key {marked}, query {i}: cosine {cosine:.4f}, visible {sees}"
+
+
+# ------------------------------------------------------------------------------------------ gated linear attention
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decays(dtype):
+    torch.manual_seed(4)
+    n, rank, channels, tau = 50, 6, 40, 16.0
+    a = rounded(torch.randn(n, rank) * 3, dtype)
+    w2 = rounded(torch.randn(channels, rank), dtype)
+    bias = torch.randn(channels) * 4
+    wide = torch.zeros(n, rank + 11, dtype=dtype)             # a view into wider rows, as the part passes it
+    wide[:, 11:] = a.to(dtype)
+    got = ops.gla_decay(wide.cuda()[:, 11:], w2.to(dtype).cuda(), bias.cuda(), tau).cpu()
+    want = torch.sigmoid(a @ w2.t() + bias).pow(1.0 / tau)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+    assert got.dtype == torch.float32 and float(got.min()) > 0.0 and float(got.max()) <= 1.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,dim,vdim", [(3, 16, 32), (1, 20, 24), (2, 64, 128), (2, 130, 70), (5, 8, 8)])
+def test_recurrence_over_entries_from_their_slots(dtype, heads, dim, vdim):
+    torch.manual_seed(5)
+    lengths, slots = [1, 37, 2, 16, 17], [3, 0, 5, 1, 4]
+    n = sum(lengths)
+    width = 2 * heads * dim + heads * vdim
+    rows = rounded(torch.randn(n, width) * 0.5, dtype)
+    alpha = torch.rand(n, heads * dim) * 0.5 + 0.5
+    state = torch.randn(6, heads, dim, vdim)
+    q, k, v = rows[:, :heads * dim], rows[:, heads * dim:2 * heads * dim], rows[:, 2 * heads * dim:]
+    want_o = torch.zeros(n, heads, vdim)
+    want_state = state.clone()
+    at = 0
+    for length, slot in zip(lengths, slots):
+        s = want_state[slot].clone()
+        for t in range(at, at + length):
+            s = alpha[t].view(heads, dim, 1) * s + k[t].view(heads, dim, 1) * v[t].view(heads, 1, vdim)
+            want_o[t] = torch.einsum("hdv,hd->hv", s, q[t].view(heads, dim) * dim ** -0.5)
+        want_state[slot] = s
+        at += length
+    device_rows = rows.to(dtype).cuda()
+    device_state = state.clone().cuda()
+    starts = torch.tensor([0] + torch.tensor(lengths).cumsum(0).tolist(), dtype=torch.int32).cuda()
+    got = ops.gla_scan(device_rows[:, :heads * dim], device_rows[:, heads * dim:2 * heads * dim],
+                       device_rows[:, 2 * heads * dim:], alpha.cuda(), starts,
+                       torch.tensor(slots, dtype=torch.int32).cuda(), device_state, dim ** -0.5)
+    torch.testing.assert_close(got.cpu(), want_o, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(device_state.cpu(), want_state, rtol=1e-4, atol=1e-4)
+    assert torch.equal(device_state[2].cpu(), state[2])       # a slot that no entry names is left alone
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_recurrence_cut_anywhere_gives_the_same_bits(dtype):
+    torch.manual_seed(6)
+    heads, dim, vdim, n = 2, 24, 40, 53
+    rows = (torch.randn(n, 2 * heads * dim + heads * vdim) * 0.5).to(dtype).cuda()
+    alpha = (torch.rand(n, heads * dim) * 0.3 + 0.7).cuda()
+
+    def run(cuts):
+        state = torch.zeros(2, heads, dim, vdim, device="cuda")
+        outs = []
+        for lo, hi in zip([0] + cuts, cuts + [n]):
+            part = rows[lo:hi].contiguous()
+            outs.append(ops.gla_scan(part[:, :heads * dim], part[:, heads * dim:2 * heads * dim], part[:, 2 * heads * dim:],
+                                     alpha[lo:hi].contiguous(), torch.tensor([0, hi - lo], dtype=torch.int32).cuda(),
+                                     torch.tensor([1], dtype=torch.int32).cuda(), state, 0.2))
+        return torch.cat(outs), state
+    whole, state = run([])
+    for cuts in ([1], [16], [17, 19], list(range(1, n))):
+        again, state_again = run(cuts)
+        assert torch.equal(again, whole) and torch.equal(state_again, state)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_head_norm_and_gate(dtype):
+    torch.manual_seed(7)
+    n, heads, vdim, eps = 19, 3, 40, 1e-5
+    o = torch.randn(n, heads, vdim) * 3
+    weight = torch.randn(vdim)
+    gate = rounded(torch.randn(n, heads * vdim) * 2, dtype)
+    got = ops.gla_norm_gate(o.cuda(), weight.cuda(), gate.to(dtype).cuda(), eps).float().cpu()
+    want = (plain.rms(o, eps) * weight).reshape(n, -1) * (gate * torch.sigmoid(gate))
+    torch.testing.assert_close(got, want, **tol(dtype))
+
+
+# ------------------------------------------------------------------------------------------ activation, soft cap
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gelu_gate_and_soft_cap(dtype):
+    torch.manual_seed(8)
+    gate_up = rounded(torch.randn(23, 2 * 56) * 3, dtype)
+    got = ops.act_mul(gate_up.to(dtype).cuda(), "gelu_tanh").float().cpu()
+    torch.testing.assert_close(got, plain.gelu_tanh(gate_up[:, :56]) * gate_up[:, 56:], **tol(dtype))
+    silu = ops.act_mul(gate_up.to(dtype).cuda(), "silu").float().cpu()
+    torch.testing.assert_close(silu, torch.nn.functional.silu(gate_up[:, :56]) * gate_up[:, 56:], **tol(dtype))
+    logits = torch.randn(7, 301) * 40
+    capped = ops.softcap_(logits.clone().cuda(), 30.0).cpu()
+    torch.testing.assert_close(capped, 30.0 * torch.tanh(logits / 30.0), rtol=1e-5, atol=1e-5)
+    assert float(capped.abs().max()) <= 30.0
