@@ -859,3 +859,58 @@ def gla_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, eps
                                         ctypes.c_int64(gate.stride(0)), ctypes.c_float(eps), _ptr(y), n, heads, vdim,
                                         _stream()))
     return y
+
+
+def diff_attention_mfma_supported(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> bool:
+    """The matrix-core kernel takes these operands: bfloat16, key and value sizes it is built for, pages of a multiple
+    of 4 keys, rows aligned to 8 bytes."""
+    return (q.dtype == torch.bfloat16 and q.shape[1] % 4 == 0 and q.data_ptr() % 8 == 0
+            and bool(library().somi_diff_attention_mfma_supported(k_cache.shape[3], v_cache.shape[2], k_cache.shape[2])))
+
+
+def diff_attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, nq: int,
+                        window: int, keep_first: int, scale: float, lam: float, eps: float, out_scale: float,
+                        out: torch.Tensor, *, entry_start: torch.Tensor | None = None,
+                        entry_first_position: torch.Tensor | None = None, entry_len: torch.Tensor | None = None,
+                        max_entry_len: int = 0, token_list: torch.Tensor | None = None,
+                        token_entry: torch.Tensor | None = None, positions: torch.Tensor | None = None) -> None:
+    """Differential attention on the matrix cores into ``out`` ([N, nq * dv] bfloat16); operands as
+    :func:`diff_attention_plain`.  Either the portions of a step (``entry_start`` [E + 1], ``entry_first_position`` [E],
+    ``max_entry_len``; ``entry_len`` [E] stands for the offsets' own lengths, 0 leaves a portion out), or listed tokens
+    (``token_entry`` and ``positions`` [N]; ``token_list`` names the tokens to run, None: all)."""
+    _need(q, "q", torch.bfloat16)
+    n = q.shape[0]
+    _need(k_cache, "k cache", torch.bfloat16)
+    _need(v_cache, "v cache", torch.bfloat16)
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.shape[1] != 2 * v_cache.shape[1]:
+        raise KernelError("diff_attention: caches must be k [pages, 2 kv_heads, page, dk] and v [pages, kv_heads, dv, page]")
+    pages, nkv, dv, page_size = v_cache.shape
+    dk = k_cache.shape[3]
+    if k_cache.shape[0] != pages or k_cache.shape[2] != page_size:
+        raise KernelError(f"diff_attention: k cache {tuple(k_cache.shape)} and v cache {tuple(v_cache.shape)} disagree")
+    if q.shape[1] < 2 * nq * dk:
+        raise KernelError("diff_attention: q rows are narrower than 2 * heads * dk")
+    _need(block_table, "block table", torch.int32)
+    _need(out, "attention out", torch.bfloat16, (n, nq * dv))
+    listed = entry_start is None
+    entries, n_list = block_table.shape[0], 0
+    if listed:
+        _need(token_entry, "token entries", torch.int32, (n,))
+        _need(positions, "positions", torch.int32, (n,))
+        n_list = n
+        if token_list is not None:
+            _need(token_list, "token list", torch.int32)
+            n_list = token_list.numel()
+    else:
+        _need(entry_start, "entry offsets", torch.int32, (entries + 1,))
+        _need(entry_first_position, "entry first positions", torch.int32, (entries,))
+        if entry_len is not None:
+            _need(entry_len, "entry lengths", torch.int32, (entries,))
+        if not 0 <= max_entry_len <= n:
+            raise KernelError(f"diff_attention: longest portion {max_entry_len} does not fit {n} tokens")
+    _check(library().somi_diff_attention_mfma(
+        _ptr(q), ctypes.c_int64(q.shape[1]), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+        1 if listed else 0, _ptr(entry_start), _ptr(entry_first_position), _ptr(entry_len), entries, int(max_entry_len),
+        _ptr(token_list), _ptr(token_entry), _ptr(positions), n_list, nq, nkv, dk, dv, page_size, int(window),
+        int(keep_first), ctypes.c_float(scale), ctypes.c_float(lam), ctypes.c_float(eps), ctypes.c_float(out_scale),
+        _ptr(out), _stream()))

@@ -106,9 +106,10 @@ def test_differential_attention_against_the_plain_maps(dtype, heads, g, dk, dv, 
     assert torch.equal(out[some.long()], got[some.long()])
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dtype,kernel", [(torch.float32, "plain"), (torch.bfloat16, "plain"),
+                                          (torch.bfloat16, "portion"), (torch.bfloat16, "listed")])
 @pytest.mark.parametrize("page,size,keep", [(16, 40, 6), (8, 33, 16), (4, 9, 2), (16, 16, 16)])
-def test_one_key_stands_out_exactly_where_the_mask_lets_it(dtype, page, size, keep):
+def test_one_key_stands_out_exactly_where_the_mask_lets_it(dtype, kernel, page, size, keep):
     """One key carries a large score against every query: a query's output is that key's value (normed) if and only
     if the key is the query itself, within the window or among the kept first tokens."""
     torch.manual_seed(3)
@@ -120,14 +121,57 @@ def test_one_key_stands_out_exactly_where_the_mask_lets_it(dtype, page, size, ke
         k[marked] = rounded(6.0 * direction, dtype)
         v = rounded(torch.randn(t, 1, dv), dtype)
         kc, vc, table = paged(k, v, page, dtype, seed=marked)
-        got = ops.diff_attention_plain(q.view(t, -1).to(dtype).cuda(), kc, vc, table,
-                                       torch.zeros(t, dtype=torch.int32).cuda(), torch.arange(t, dtype=torch.int32).cuda(),
-                                       1, size, keep, 1.0, 0.0, 1e-6, 1.0).float().cpu()
+        if kernel == "plain":
+            got = ops.diff_attention_plain(q.view(t, -1).to(dtype).cuda(), kc, vc, table,
+                                           torch.zeros(t, dtype=torch.int32).cuda(),
+                                           torch.arange(t, dtype=torch.int32).cuda(),
+                                           1, size, keep, 1.0, 0.0, 1e-6, 1.0).float().cpu()
+        else:
+            got = run_matrix_core(kernel, q, kc, vc, table, 1, size, keep, 1.0, 0.0, 1e-6, 1.0)
         marked_value = plain.rms(v[marked, 0], 1e-6)
         for i in range(t):
             sees = plain.visible(i, marked, size, keep)
             cosine = float(torch.nn.functional.cosine_similarity(got[i], marked_value, dim=0))
             assert (cosine > 0.999) == sees, f"key {marked}, query {i}: cosine {cosine:.4f}, visible {sees}"
+
+
+def run_matrix_core(kind, q, kc, vc, table, heads, size, keep, scale, lam, eps, out_scale, first=0):
+    """The matrix-core kernel on the tokens at positions first .. first + len(q) - 1 of the one request whose pages
+    ``table`` lists: as one portion, or as listed tokens."""
+    n = q.shape[0]
+    flat = q.reshape(n, -1).to(torch.bfloat16).cuda()
+    out = torch.zeros((n, heads * vc.shape[2]), dtype=torch.bfloat16, device="cuda")
+    args = (flat, kc, vc, table, heads, size, keep, scale, lam, eps, out_scale, out)
+    if kind == "portion":
+        ops.diff_attention_mfma(*args, entry_start=torch.tensor([0, n], dtype=torch.int32).cuda(),
+                                entry_first_position=torch.tensor([first], dtype=torch.int32).cuda(), max_entry_len=n)
+    else:
+        ops.diff_attention_mfma(*args, token_entry=torch.zeros(n, dtype=torch.int32).cuda(),
+                                positions=torch.arange(first, first + n, dtype=torch.int32).cuda())
+    return out.float().cpu()
+
+
+@pytest.mark.parametrize("kind", ["portion", "listed"])
+@pytest.mark.parametrize("heads,g,dk,dv,page,t,size,keep", [
+    (4, 2, 16, 32, 16, 150, 24, 5), (3, 1, 48, 32, 16, 300, 130, 17), (4, 4, 32, 16, 32, 260, 128, 128),
+    (8, 2, 64, 128, 8, 200, 50, 3), (2, 1, 16, 16, 4, 90, 7, 9), (16, 1, 128, 64, 16, 70, 1000, 0),
+    (6, 1, 32, 48, 16, 130, 33, 40)])
+def test_matrix_core_kernel_against_the_plain_maps(kind, heads, g, dk, dv, page, t, size, keep):
+    dtype = torch.bfloat16
+    torch.manual_seed(9)
+    q = rounded(torch.randn(t, 2 * heads, dk), dtype)
+    k = rounded(torch.randn(t, 2 * g, dk), dtype)
+    v = rounded(torch.randn(t, g, dv), dtype)
+    kc, vc, table = paged(k, v, page, dtype, seed=t)
+    assert ops.diff_attention_mfma_supported(q.view(t, -1).to(dtype).cuda(), kc, vc)
+    scale, lam, eps, out_scale = 0.4, 0.55, 1e-5, 0.7
+    want = plain_differential(q, k, v, heads, scale, size, keep, lam, eps, out_scale)
+    got = run_matrix_core(kind, q, kc, vc, table, heads, size, keep, scale, lam, eps, out_scale)
+    torch.testing.assert_close(got, want, **tol(dtype))
+    # the last tokens alone, from what is cached: a portion that starts in the middle of a page, a window and a tile
+    for first in (t - 1, t - 7, t // 2 + 3):
+        part = run_matrix_core(kind, q[first:], kc, vc, table, heads, size, keep, scale, lam, eps, out_scale, first=first)
+        torch.testing.assert_close(part, want[first:], **tol(dtype))
 
 
 # ------------------------------------------------------------------------------------------ gated linear attention
