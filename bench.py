@@ -48,6 +48,41 @@ LAYER_SIZES = {
     "14b": (48, 5120, 40, 8, 128, 13824, 1e-5, 152064, False),
     "32b": (64, 5120, 40, 8, 128, 27648, 1e-6, 152064, False),
 }
+# layer sizes of Kamedra models that resemble real ones: (width, feed-forward, attention heads, key/value heads, size
+# of one query/key map, value size, recurrent heads, their key size, their value size, rank of the decay's projection,
+# window, kept first tokens, vocabulary).  Six layers: two recurrent ones, attention with a feed-forward, two recurrent
+# ones, attention that borrows the first one's keys and values with a feed-forward.
+KAMEDRA_SIZES = {
+    "1b": (2048, 8192, 16, 4, 64, 128, 16, 64, 128, 64, 1024, 4, 32000),
+    "7b": (4096, 14336, 32, 8, 64, 128, 32, 64, 128, 64, 2048, 4, 32000),
+}
+
+
+def kamedra_config_dict(sizes: str) -> dict:
+    width, ff, heads, kv_heads, dim, vdim, r_heads, r_dim, r_vdim, rank, window, keep, vocab = KAMEDRA_SIZES[sizes]
+    recurrent = {"type": "gla", "mlp": None, "mixer": {"heads": r_heads, "dim": r_dim, "vdim": r_vdim, "tau": 16.0, "rank": rank}}
+
+    def attention(kv_from=None):
+        mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "diff": 0.6, "scale": dim ** -0.5,
+                 "mask": {"size": window, "keep_first": keep},
+                 "rot": {"base": 500000.0, "dims": dim, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+        if kv_from is not None:
+            mixer["kv_from"] = kv_from
+        return {"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}}
+    return {"architecture": "Kamedra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+            "layers": [recurrent, recurrent, attention(), recurrent, recurrent, attention(2)]}
+
+
+def closest_config_dict(sizes: str) -> dict:
+    """The Qwen2.5-style model of the same width, heads (one head of twice the map size for a head's two maps),
+    key/value heads, feed-forward, vocabulary and number of layers."""
+    width, ff, heads, kv_heads, dim, _, _, _, _, _, _, _, vocab = KAMEDRA_SIZES[sizes]
+    return {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "vocab_size": vocab, "hidden_size": width,
+            "intermediate_size": ff, "num_hidden_layers": 6, "num_attention_heads": heads,
+            "num_key_value_heads": kv_heads, "head_dim": 2 * dim, "rope_theta": 5e5, "rms_norm_eps": 1e-6,
+            "tie_word_embeddings": True, "max_position_embeddings": 32768, "hidden_act": "silu", "attention_bias": False}
+
+
 # keys of a config.json that name sizes, in the order they are reported under "config" (flat, at most 20 keys)
 SIZE_KEYS = ("hidden_size", "intermediate_size", "num_attention_heads", "num_key_value_heads", "head_dim",
              "vocab_size", "tie_word_embeddings")
@@ -80,6 +115,10 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--stages", action="store_true",
                    help="also time the named stages of an eager prefill and an eager decode step and report their shares")
     p.add_argument("--output-file", type=str, default=None, help="Append the result line to a JSONL file.")
+    p.add_argument("--kamedra", default=None, choices=sorted(KAMEDRA_SIZES), metavar="SIZES",
+                   help="instead of the default workload: prefill and decode of a Kamedra model (differential attention "
+                        "with a window, gated linear attention) at these layer sizes, beside the Qwen2.5-style model of "
+                        "equal width, heads, feed-forward and layers, each with its stage times")
     p.add_argument("--serving", type=int, default=0, metavar="REQUESTS",
                    help="also run this many requests (prompts of 128 to 2,048 tokens, 256 new tokens each) through "
                         "the scheduler with portions of 512, and report it under 'serving'")
@@ -454,6 +493,63 @@ def run_extras(args, started: float) -> dict:
     return extras
 
 
+def run_kamedra(args) -> dict:
+    """Prefill and decode of a Kamedra model beside the closest Qwen2.5-style model, with the stage times of both and
+    what the attention and recurrence stages reach of the machine."""
+    width, ff, heads, kv_heads, dim, vdim, r_heads, r_dim, r_vdim, rank, window, keep, vocab = KAMEDRA_SIZES[args.kamedra]
+    batches, context, tokens = (8, 64), args.context, args.prefill_tokens
+    out: dict = {}
+    for label, config_dict in (("kamedra", kamedra_config_dict(args.kamedra)), ("closest", closest_config_dict(args.kamedra))):
+        bench = Workbench(config_dict, dtype=args.dtype, seed=args.seed, block_size=args.block_size,
+                          pool_tokens=Workbench.pool_tokens(batches, context, tokens), max_requests=max(batches))
+        block: dict = {"prefill": {str(n): bench.prefill_run(n) for n in sorted({512, tokens})}}
+        for batch in batches:
+            run = bench.decode_run(batch, max(POINT_MIN_STEPS, args.steps // 2), max(2, args.warmup // 2), context)
+            block[f"decode_b{batch}"] = {"tok_s": round(run["tok_s"], 1), "ms": round(run["ms"], 4),
+                                        "mean_ctx": round(run["mean_ctx"], 1)}
+        block["stages"] = bench.stage_run(tokens, batches[0], context)
+        print_stage_tables(block["stages"])
+        out[label] = block
+        bench.close()
+    # what the mixers' own kernels reach: matrix operations of a prefill's attention (both maps' scores and both
+    # maps' weights times values over the visible pairs; causal pairs for the closest model) and of the recurrence
+    bf16_peak = PEAK_FLOPS["bfloat16"]
+    pairs_window = sum(min(p + 1, window + (keep if p >= window else 0)) for p in range(tokens))
+    pairs_causal = tokens * (tokens + 1) // 2
+
+    def stage_ms(block, run, name):
+        return block["stages"][run].get(name, {}).get("ms", 0.0)
+    run = f"prefill_{tokens}"
+    k_ms, c_ms = stage_ms(out["kamedra"], run, "attention"), stage_ms(out["closest"], run, "attention")
+    r_ms = stage_ms(out["kamedra"], run, "recurrence")
+    k_flops = 2 * 4.0 * heads * (dim + vdim) * pairs_window           # two attention layers
+    c_flops = 6 * 4.0 * heads * (2 * dim) * pairs_causal              # six attention layers
+    r_flops = 4 * 4.0 * r_heads * r_dim * r_vdim * tokens             # four recurrent layers
+    out["prefill_kernels"] = {
+        "tokens": tokens,
+        "kamedra_attention": {"ms": k_ms, "tflops": round(k_flops / 1e9 / max(k_ms, 1e-9), 2),
+                              "frac_of_peak": round(k_flops / 1e3 / max(k_ms, 1e-9) / bf16_peak * 1e6, 5)},
+        "closest_attention": {"ms": c_ms, "tflops": round(c_flops / 1e9 / max(c_ms, 1e-9), 2),
+                              "frac_of_peak": round(c_flops / 1e3 / max(c_ms, 1e-9) / bf16_peak * 1e6, 5)},
+        "kamedra_recurrence": {"ms": r_ms, "tflops": round(r_flops / 1e9 / max(r_ms, 1e-9), 3)},
+    }
+    # a decode step's attention reads the visible keys and values; its recurrence reads and writes the states
+    run = f"decode_b{batches[0]}_eager"
+    k_ms, c_ms = stage_ms(out["kamedra"], run, "attention"), stage_ms(out["closest"], run, "attention")
+    r_ms = stage_ms(out["kamedra"], run, "recurrence")
+    seen = min(context, window + keep)
+    k_bytes = 2 * batches[0] * seen * kv_heads * (2 * dim + vdim) * 2.0
+    c_bytes = 6 * batches[0] * context * kv_heads * (2 * 2 * dim) * 2.0
+    r_bytes = 4 * batches[0] * r_heads * r_dim * r_vdim * 4.0 * 2
+    out["decode_kernels"] = {
+        "batch": batches[0], "context": context,
+        "kamedra_attention": {"ms": k_ms, "gbs": round(k_bytes / 1e6 / max(k_ms, 1e-9), 1)},
+        "closest_attention": {"ms": c_ms, "gbs": round(c_bytes / 1e6 / max(c_ms, 1e-9), 1)},
+        "kamedra_recurrence": {"ms": r_ms, "gbs": round(r_bytes / 1e6 / max(r_ms, 1e-9), 1)},
+    }
+    return out
+
+
 def main() -> int:
     args = parse_args()
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -462,6 +558,15 @@ def main() -> int:
             print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} (WORLD_SIZE {world}) is not supported")
         return 2
     started = time.perf_counter()
+    if args.kamedra:
+        line = {"metric": f"Kamedra at {args.kamedra} layer sizes beside the closest Qwen2.5-style model: prefill and decode",
+                "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                "data": "synthetic: seeded random weights, seeded uniform token ids", "sizes": args.kamedra}
+        line.update(run_kamedra(args))
+        line["value"] = line["kamedra"][f"decode_b8"]["tok_s"]
+        line["seconds_total"] = round(time.perf_counter() - started, 1)
+        print(json.dumps(line))
+        return 0
 
     import torch
 

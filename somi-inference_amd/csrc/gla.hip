@@ -1,6 +1,7 @@
 // Gated linear attention: a recurrent state per request and head, carried from token to token.
 //
-//   alpha[t, h, d] = sigmoid(z)^(1/tau),  z = W2 (a[t]) + b           (a: the low-rank projection of the input)
+//   alpha[t, h, d] = sigmoid(z)^(1/tau),  z = W2 (a[t]) + b           (a: the low-rank projection of the input; z
+//                                                                    comes from the engine's matrix products)
 //   S_t[d, c]      = alpha[t, h, d] * S_(t-1)[d, c] + k[t, h, d] * v[t, h, c]          S: [dim, vdim] per head
 //   o[t, h, c]     = sum_d S_t[d, c] * q[t, h, d] * q_scale
 //   y[t, h, c]     = o / sqrt(mean_c(o^2) + eps) * w[c] * silu(g[t, h, c])
@@ -13,53 +14,37 @@
 #include "common.h"
 
 // ------------------------------------------------------------------------------------------------ decays
-// alpha[t, c] = exp(-softplus(-z) / tau), z = bias[c] + sum_r a[t, r] * w2[c, r].  One thread per (t, c).
-template <typename T>
+// alpha = sigmoid(z)^(1 / tau) = exp(-softplus(-z) / tau), in place on the float32 sums z of the decay's projection.
 __global__ void __launch_bounds__(256)
-gla_decay_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w2, const float* __restrict__ bias,
-                 float inv_tau, float* __restrict__ alpha, int channels, int rank, int64_t count) {
+gla_alpha_kernel(float* __restrict__ z, float inv_tau, int64_t count) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256) {
-        const int64_t t = i / channels;
-        const int c = (int)(i - t * channels);
-        const T* ar = a + t * a_stride;
-        const T* wr = w2 + (int64_t)c * rank;
-        float z = 0.f;
-        for (int r = 0; r < rank; ++r) z = fmaf(to_float(ar[r]), to_float(wr[r]), z);
-        z += bias ? bias[c] : 0.f;
-        // log sigmoid(z) = -softplus(-z) = -(max(-z, 0) + log1p(exp(-|z|)))
-        const float log_sigmoid = -(fmaxf(-z, 0.f) + log1pf(expf(-fabsf(z))));
-        alpha[i] = expf(log_sigmoid * inv_tau);
+        const float x = z[i];
+        // log sigmoid(x) = -softplus(-x) = -(max(-x, 0) + log1p(exp(-|x|)))
+        const float log_sigmoid = -(fmaxf(-x, 0.f) + log1pf(expf(-fabsf(x))));
+        z[i] = expf(log_sigmoid * inv_tau);
     }
 }
 
-extern "C" int somi_gla_decay(const void* a, int dtype, int64_t a_stride, const void* w2, const float* bias, float tau,
-                              float* alpha, int n_tokens, int channels, int rank, hipStream_t stream) {
-    SOMI_REQUIRE(n_tokens >= 0 && channels > 0 && rank > 0 && a_stride >= rank, "gla_decay: bad sizes");
-    SOMI_REQUIRE(tau > 0.f, "gla_decay: tau must be > 0");
-    const int64_t count = (int64_t)n_tokens * channels;
+extern "C" int somi_gla_alpha(float* z, float tau, int64_t count, hipStream_t stream) {
+    SOMI_REQUIRE(count >= 0 && tau > 0.f, "gla_alpha: bad arguments");
     if (count == 0) return 0;
     const int grid = (int)(ceil_div64(count, 256) < 65536 ? ceil_div64(count, 256) : 65536);
-    if (dtype == SOMI_F32)
-        hipLaunchKernelGGL(gla_decay_kernel<float>, dim3(grid), dim3(256), 0, stream, (const float*)a, a_stride,
-                           (const float*)w2, bias, 1.0f / tau, alpha, channels, rank, count);
-    else if (dtype == SOMI_BF16)
-        hipLaunchKernelGGL(gla_decay_kernel<bf16>, dim3(grid), dim3(256), 0, stream, (const bf16*)a, a_stride,
-                           (const bf16*)w2, bias, 1.0f / tau, alpha, channels, rank, count);
-    else
-        return somi_fail("gla_decay: unknown dtype %d", dtype);
-    SOMI_LAUNCH_CHECK("gla_decay");
+    hipLaunchKernelGGL(gla_alpha_kernel, dim3(grid), dim3(256), 0, stream, z, 1.0f / tau, count);
+    SOMI_LAUNCH_CHECK("gla_alpha");
     return 0;
 }
 
 // ------------------------------------------------------------------------------------------------ the recurrence
-// A wavefront owns GLA_COLS columns of one (entry, head): lane = column + GLA_COLS * row group; row group r of
-// GLA_GROUPS holds the rows d = r, r + GLA_GROUPS, ... of its column in registers (RPL of them).  Per token the
-// wavefront's alpha, k and q of the head are staged through LDS GLA_STAGE tokens at a time (a workgroup is one wavefront, which
-// stages for itself), a lane updates its rows and sums its share of o, and the row groups'
-// shares are added by two lane exchanges, always in the same order.
+// A wavefront (a workgroup of its own) owns GLA_COLS columns of one (entry, head): lane = column + GLA_COLS * row
+// group, and row group g of the four holds the rows d = g * RPL .. g * RPL + RPL - 1 of its column in registers (rows
+// past dim are padding that stays zero).  The tokens' alpha, k and scaled q of the head go through LDS STAGE tokens at
+// a time, laid out so that a lane reads its rows four at a time; the next tokens' values are asked of memory before
+// the staged ones are worked on, so a token costs no memory latency.  Per token a lane updates its rows, sums its share
+// of o, and the row groups' shares are added by two lane exchanges, always in the same order.
 #define GLA_COLS 16
 #define GLA_GROUPS 4
-#define GLA_STAGE 16
+
+typedef __attribute__((ext_vector_type(4))) float gla_f32x4;
 
 template <typename T, int RPL>
 __global__ void __launch_bounds__(64)
@@ -67,7 +52,12 @@ gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __res
                 const float* __restrict__ alpha, const int* __restrict__ entry_start,
                 const int* __restrict__ state_slots, float* __restrict__ state, int heads, int dim, int vdim,
                 float q_scale, float* __restrict__ o) {
-    extern __shared__ float staged[];              // [3][GLA_STAGE][dim]: alpha, k, q (scaled)
+    constexpr int STAGE = RPL <= 16 ? 16 : (RPL <= 32 ? 8 : 4);       // tokens staged at a time
+    constexpr int ROWS = GLA_GROUPS * RPL;                             // padded rows of a head
+    constexpr int PER_LANE = STAGE * ROWS / 64;                        // staged elements of each array a lane moves
+    __shared__ __attribute__((aligned(16))) float sa[STAGE * ROWS];
+    __shared__ __attribute__((aligned(16))) float sk[STAGE * ROWS];
+    __shared__ __attribute__((aligned(16))) float sq[STAGE * ROWS];
     const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int col = blockIdx.z * GLA_COLS + (lane % GLA_COLS), group = lane / GLA_COLS;
     const bool live = col < vdim;
@@ -76,45 +66,68 @@ gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __res
     float s[RPL];
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
-        const int d = group + i * GLA_GROUPS;
+        const int d = group * RPL + i;
         s[i] = (live && d < dim) ? S[(int64_t)d * vdim + col] : 0.f;
     }
-    float* sa = staged;
-    float* sk = staged + GLA_STAGE * dim;
-    float* sq = staged + 2 * GLA_STAGE * dim;
-    for (int base = t0; base < t1; base += GLA_STAGE) {
-        const int count = min(GLA_STAGE, t1 - base);
-        for (int i = lane; i < count * dim; i += 64) {
-            const int tt = i / dim, d = i - tt * dim;
-            const int64_t at = (int64_t)(base + tt) * row_stride + (int64_t)h * dim + d;
-            sa[i] = alpha[((int64_t)(base + tt) * heads + h) * dim + d];
-            sk[i] = to_float(k[at]);
-            sq[i] = to_float(q[at]) * q_scale;
-        }
-        __syncthreads();                           // one wavefront a workgroup: its stores to LDS before its reads
-        for (int tt = 0; tt < count; ++tt) {
-            const float vt = live ? to_float(v[(int64_t)(base + tt) * row_stride + (int64_t)h * vdim + col]) : 0.f;
-            const float* a = sa + tt * dim;
-            const float* kk = sk + tt * dim;
-            const float* qq = sq + tt * dim;
-            float acc = 0.f;
+    float na[PER_LANE], nk[PER_LANE], nq[PER_LANE], nv[STAGE];        // the next tokens, on their way from memory
+
+    auto fetch = [&](int base) {
 #pragma unroll
-            for (int i = 0; i < RPL; ++i) {
-                const int d = group + i * GLA_GROUPS;
-                if (d < dim) {
-                    s[i] = fmaf(a[d], s[i], kk[d] * vt);
-                    acc = fmaf(s[i], qq[d], acc);
+        for (int j = 0; j < PER_LANE; ++j) {
+            const int el = lane + 64 * j, tt = el / ROWS, d = el % ROWS, t = base + tt;
+            const bool there = t < t1 && d < dim;
+            const int64_t at = (int64_t)t * row_stride + (int64_t)h * dim + d;
+            na[j] = there ? alpha[((int64_t)t * heads + h) * dim + d] : 0.f;
+            nk[j] = there ? to_float(k[at]) : 0.f;
+            nq[j] = there ? to_float(q[at]) * q_scale : 0.f;
+        }
+#pragma unroll
+        for (int tt = 0; tt < STAGE; ++tt)
+            nv[tt] = (live && base + tt < t1) ? to_float(v[(int64_t)(base + tt) * row_stride + (int64_t)h * vdim + col]) : 0.f;
+    };
+
+    if (t0 < t1) fetch(t0);
+    for (int base = t0; base < t1; base += STAGE) {
+        const int count = min(STAGE, t1 - base);
+        float vt[STAGE];
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) {
+            sa[lane + 64 * j] = na[j];
+            sk[lane + 64 * j] = nk[j];
+            sq[lane + 64 * j] = nq[j];
+        }
+#pragma unroll
+        for (int tt = 0; tt < STAGE; ++tt) vt[tt] = nv[tt];
+        __syncthreads();                           // one wavefront a workgroup: its stores to LDS before its reads
+        if (base + STAGE < t1) fetch(base + STAGE);
+#pragma unroll
+        for (int tt = 0; tt < STAGE; ++tt) {
+            if (tt < count) {
+                const float* a = sa + tt * ROWS + group * RPL;
+                const float* kk = sk + tt * ROWS + group * RPL;
+                const float* qq = sq + tt * ROWS + group * RPL;
+                float acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < RPL; i += 4) {
+                    const gla_f32x4 a4 = *reinterpret_cast<const gla_f32x4*>(a + i);
+                    const gla_f32x4 k4 = *reinterpret_cast<const gla_f32x4*>(kk + i);
+                    const gla_f32x4 q4 = *reinterpret_cast<const gla_f32x4*>(qq + i);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        s[i + x] = fmaf(a4[x], s[i + x], k4[x] * vt[tt]);
+                        acc = fmaf(s[i + x], q4[x], acc);
+                    }
                 }
+                acc += __shfl_xor(acc, GLA_COLS, 64);
+                acc += __shfl_xor(acc, 2 * GLA_COLS, 64);
+                if (live && group == 0) o[((int64_t)(base + tt) * heads + h) * vdim + col] = acc;
             }
-            acc += __shfl_xor(acc, GLA_COLS, 64);
-            acc += __shfl_xor(acc, 2 * GLA_COLS, 64);
-            if (live && group == 0) o[((int64_t)(base + tt) * heads + h) * vdim + col] = acc;
         }
         __syncthreads();                           // the reads, before the next tokens are staged
     }
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
-        const int d = group + i * GLA_GROUPS;
+        const int d = group * RPL + i;
         if (live && d < dim) S[(int64_t)d * vdim + col] = s[i];
     }
 }
@@ -133,16 +146,19 @@ extern "C" int somi_gla_scan(const void* q, const void* k, const void* v, int dt
     SOMI_REQUIRE(heads <= 65535 && ceil_div(vdim, GLA_COLS) <= 65535, "gla_scan: too many heads or columns");
     if (n_entries == 0) return 0;
     const dim3 grid(n_entries, heads, ceil_div(vdim, GLA_COLS));
-    const size_t lds = (size_t)3 * GLA_STAGE * dim * sizeof(float);
     const int rpl = ceil_div(dim, GLA_GROUPS);
 #define GLA_LAUNCH(T, R)                                                                                              \
-    hipLaunchKernelGGL((gla_scan_kernel<T, R>), grid, dim3(64), lds, stream, (const T*)q, (const T*)k, (const T*)v,   \
+    hipLaunchKernelGGL((gla_scan_kernel<T, R>), grid, dim3(64), 0, stream, (const T*)q, (const T*)k, (const T*)v,     \
                        row_stride, alpha, entry_start, state_slots, state, heads, dim, vdim, q_scale, o)
 #define GLA_BY_ROWS(T)                                                                                                \
     do {                                                                                                              \
-        if (rpl <= 8) GLA_LAUNCH(T, 8);                                                                               \
+        if (rpl <= 4) GLA_LAUNCH(T, 4);                                                                               \
+        else if (rpl <= 8) GLA_LAUNCH(T, 8);                                                                          \
+        else if (rpl <= 12) GLA_LAUNCH(T, 12);                                                                        \
         else if (rpl <= 16) GLA_LAUNCH(T, 16);                                                                        \
+        else if (rpl <= 24) GLA_LAUNCH(T, 24);                                                                        \
         else if (rpl <= 32) GLA_LAUNCH(T, 32);                                                                        \
+        else if (rpl <= 48) GLA_LAUNCH(T, 48);                                                                        \
         else GLA_LAUNCH(T, 64);                                                                                       \
     } while (0)
     if (dtype == SOMI_F32) GLA_BY_ROWS(float);

@@ -161,8 +161,8 @@ class ModelRunner:
         slots = static.batch.state_slots.to(torch.int64) if stateful else None
         before = [cache.state.index_select(0, slots) for cache in stateful]
         self.model.forward(static.batch, self.cache.layer_caches)
-        for cache, rows in zip(stateful, before):
-            cache.state.index_copy_(0, slots, rows)
+        for cache, saved in zip(stateful, before):
+            cache.state.index_copy_(0, slots, saved)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):

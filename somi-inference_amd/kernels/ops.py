@@ -804,22 +804,11 @@ def diff_attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
     return out
 
 
-def gla_decay(a: torch.Tensor, w2: torch.Tensor, bias: torch.Tensor | None, tau: float) -> torch.Tensor:
-    """alpha = sigmoid(a @ w2.T + bias)^(1 / tau) in float32 -> [N, channels].  a: [N, rank] (a view with a row stride of
-    its own is taken as it is); w2: [channels, rank]."""
-    if not isinstance(a, torch.Tensor) or not a.is_cuda or a.dim() != 2 or a.stride(1) != 1:
-        raise KernelError("gla_decay: the input must be a matrix on the GPU with contiguous rows")
-    n, rank = a.shape
-    _need(w2, "decay weight", a.dtype)
-    if w2.dim() != 2 or w2.shape[1] != rank:
-        raise KernelError(f"gla_decay: weight {tuple(w2.shape)} does not fit a rank of {rank}")
-    channels = w2.shape[0]
-    if bias is not None:
-        _need(bias, "decay bias", torch.float32, (channels,))
-    alpha = torch.empty((n, channels), dtype=torch.float32, device=a.device)
-    _check(library().somi_gla_decay(_ptr(a), dtype_code(a.dtype), ctypes.c_int64(a.stride(0)), _ptr(w2), _ptr(bias),
-                                    ctypes.c_float(tau), _ptr(alpha), n, channels, rank, _stream()))
-    return alpha
+def gla_alpha_(z: torch.Tensor, tau: float) -> torch.Tensor:
+    """z <- sigmoid(z)^(1 / tau), in place on float32 values (through the logarithm: exp(-softplus(-z) / tau))."""
+    _need(z, "decay sums", torch.float32)
+    _check(library().somi_gla_alpha(_ptr(z), ctypes.c_float(tau), ctypes.c_int64(z.numel()), _stream()))
+    return z
 
 
 def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, alpha: torch.Tensor, entry_start: torch.Tensor,

@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import torch
 
+from ..kernels import linear as linear_kernels
 from ..kernels import ops
 from ..kernels.stages import stage
 from ..weights.spec import ANY_SIZE, MATRIX, VECTOR, Init, WeightSpec
@@ -98,7 +99,9 @@ class GatedLinearAttention(Mixer):
         q, k = rows[:, :qk], rows[:, qk:2 * qk]
         v, g = rows[:, 2 * qk:2 * qk + vv], rows[:, 2 * qk + vv:2 * qk + 2 * vv]
         with stage("decays"):
-            alpha = ops.gla_decay(rows[:, 2 * qk + 2 * vv:], self.a2, self.a2_bias, self.tau)
+            # the second matrix of the decay's projection (float32 sums and bias), then sigmoid^(1/tau) in float32
+            z = linear_kernels.linear(rows[:, 2 * qk + 2 * vv:].contiguous(), self.a2, self.a2_bias, torch.float32)
+            alpha = ops.gla_alpha_(z, self.tau)
         with stage("recurrence"):
             o = ops.gla_scan(q, k, v, alpha, step.entry_start, step.state_slots, cache.state, self.key_dim ** -0.5)
         with stage("norm, gate"):

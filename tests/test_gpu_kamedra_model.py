@@ -96,7 +96,8 @@ def test_prompt_then_long_decoding_token_by_token(name, dtype, folders, oracle):
         if dtype == "float32":
             whole = run_portions(runner, "w", tokens, [prefill + decoded])
             assert torch.equal(got, whole), "float32 logits differ between decoding and the whole prompt"
-    assert runner.graph_replays > 0          # decoded tokens took the captured step
+    assert runner.graph_replays > 0          # decoded tokens took the captured step ...
+    assert len(runner._graphs) <= 4          # ... which is captured once per shape, not once per step
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

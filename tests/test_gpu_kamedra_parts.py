@@ -175,23 +175,18 @@ def test_matrix_core_kernel_against_the_plain_maps(kind, heads, g, dk, dv, page,
 
 
 # ------------------------------------------------------------------------------------------ gated linear attention
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_decays(dtype):
+def test_decays():
     torch.manual_seed(4)
-    n, rank, channels, tau = 50, 6, 40, 16.0
-    a = rounded(torch.randn(n, rank) * 3, dtype)
-    w2 = rounded(torch.randn(channels, rank), dtype)
-    bias = torch.randn(channels) * 4
-    wide = torch.zeros(n, rank + 11, dtype=dtype)             # a view into wider rows, as the part passes it
-    wide[:, 11:] = a.to(dtype)
-    got = ops.gla_decay(wide.cuda()[:, 11:], w2.to(dtype).cuda(), bias.cuda(), tau).cpu()
-    want = torch.sigmoid(a @ w2.t() + bias).pow(1.0 / tau)
-    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
-    assert got.dtype == torch.float32 and float(got.min()) > 0.0 and float(got.max()) <= 1.0
+    z = torch.cat([torch.randn(50, 40) * 6, torch.tensor([[-80.0, -20.0, 0.0, 20.0, 80.0] * 8])])
+    for tau in (16.0, 1.0, 0.5):
+        got = ops.gla_alpha_(z.clone().cuda(), tau).cpu()
+        want = torch.sigmoid(z.double()).pow(1.0 / tau).float()
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-30)
+        assert float(got.min()) >= 0.0 and float(got.max()) <= 1.0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,dim,vdim", [(3, 16, 32), (1, 20, 24), (2, 64, 128), (2, 130, 70), (5, 8, 8)])
+@pytest.mark.parametrize("heads,dim,vdim", [(3, 16, 32), (1, 20, 24), (2, 64, 128), (2, 130, 70), (5, 8, 8), (2, 48, 64), (1, 256, 16), (2, 96, 40)])
 def test_recurrence_over_entries_from_their_slots(dtype, heads, dim, vdim):
     torch.manual_seed(5)
     lengths, slots = [1, 37, 2, 16, 17], [3, 0, 5, 1, 4]
