@@ -107,9 +107,7 @@ diff_attention_mfma_kernel(const DiffArgs a) {
         for (int c = 0; c < DVT; ++c) acc[map][c] = dmf_f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int last_block = a.max_blocks - 1;
-    // The fragments of a key tile: both maps' key rows and the value channels.  A wavefront asks for its next tile's
-    // before it works on this one's, so the products do not wait for memory.
-    auto load_tile = [&](int idx, dmf_short4 (&kf)[2][DKT], dmf_short4 (&vf)[DVT]) {
+    for (int idx = wave; idx < tiles; idx += DMF_WAVES) {
         const int tile = idx < sink_tiles ? idx : w0 + (idx - sink_tiles);
         const int j0 = tile << 4;
         // keys: lane reads row j0 + r of both maps (a row of the request's pages also where the key is masked)
@@ -121,6 +119,7 @@ diff_attention_mfma_kernel(const DiffArgs a) {
         const int vpos = min(j0 + 4 * g, pmax & ~3);
         const int64_t vpage = table[min(vpos / a.page_size, last_block)];
         const bf16* vbase = a.vc + (vpage * a.nkv + kvh) * (int64_t)DV * a.page_size + vpos % a.page_size;
+        dmf_short4 kf[2][DKT], vf[DVT];
 #pragma unroll
         for (int map = 0; map < 2; ++map)
 #pragma unroll
@@ -137,20 +136,6 @@ diff_attention_mfma_kernel(const DiffArgs a) {
                 for (int c = 0; c < DVT; ++c) vf[c][i] = 0;
             }
         }
-    };
-    dmf_short4 kf_next[2][DKT], vf_next[DVT];
-    if (wave < tiles) load_tile(wave, kf_next, vf_next);
-    for (int idx = wave; idx < tiles; idx += DMF_WAVES) {
-        const int tile = idx < sink_tiles ? idx : w0 + (idx - sink_tiles);
-        const int j0 = tile << 4;
-        dmf_short4 kf[2][DKT], vf[DVT];
-#pragma unroll
-        for (int map = 0; map < 2; ++map)
-#pragma unroll
-            for (int kk = 0; kk < DKT; ++kk) kf[map][kk] = kf_next[map][kk];
-#pragma unroll
-        for (int c = 0; c < DVT; ++c) vf[c] = vf_next[c];
-        if (idx + DMF_WAVES < tiles) load_tile(idx + DMF_WAVES, kf_next, vf_next);
 
         dmf_short4 p_hi[2], p_lo[2];
         float corr[2];

@@ -35,18 +35,41 @@ extern "C" int somi_gla_alpha(float* z, float tau, int64_t count, hipStream_t st
 }
 
 // ------------------------------------------------------------------------------------------------ the recurrence
-// A wavefront (a workgroup of its own) owns GLA_COLS columns of one (entry, head): lane = column + GLA_COLS * row
-// group, and row group g of the four holds the rows d = g * RPL .. g * RPL + RPL - 1 of its column in registers (rows
-// past dim are padding that stays zero).  The tokens' alpha, k and scaled q of the head go through LDS STAGE tokens at
-// a time, laid out so that a lane reads its rows four at a time; the next tokens' values are asked of memory before
-// the staged ones are worked on, so a token costs no memory latency.  Per token a lane updates its rows, sums its share
-// of o, and the row groups' shares are added by two lane exchanges, always in the same order.
+// A wavefront (a workgroup of its own) owns GLA_COLS columns of one (entry, head): lane = 4 * column + row group, and
+// row group g of the four holds the rows d = g * RPL .. g * RPL + RPL - 1 of its column in registers (rows past dim are
+// padding that stays zero).  The tokens' alpha, k, scaled q and v of the head go through LDS STAGE tokens at a time,
+// laid out so that a lane reads its rows four at a time.  The next tokens' values are asked of memory, as they are
+// stored (no arithmetic touches them, so nothing waits for them), before the staged ones are worked on; they are
+// converted on their way into LDS.  Per token a lane updates its rows and sums its share of o, the row groups' shares
+// are added by two exchanges inside the column's four lanes, always in the same order, and the stage's o leaves
+// through LDS in whole rows.
 #define GLA_COLS 16
 #define GLA_GROUPS 4
 
 typedef __attribute__((ext_vector_type(4))) float gla_f32x4;
 
-template <typename T, int RPL>
+// The value of another lane of the same group of four lanes (a data-parallel move: no LDS, no wait).
+template <int PATTERN> __device__ __forceinline__ float quad_swap(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), PATTERN, 0xF, 0xF, true));
+}
+
+// G consecutive elements as they are stored.
+template <typename T, int G> struct GlaRaw { T v[G]; };
+template <typename T, int G> __device__ __forceinline__ GlaRaw<T, G> gla_load(const T* p) {
+    GlaRaw<T, G> out;
+    if (G == 4) {
+        typedef __attribute__((ext_vector_type(4))) T vec4;
+        const vec4 x = *reinterpret_cast<const vec4*>(p);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out.v[i] = x[i];
+    } else {
+        out.v[0] = p[0];
+    }
+    return out;
+}
+
+// G: elements moved at a time, 4 where dim, vdim and the row strides are multiples of 4 and the rows aligned, else 1.
+template <typename T, int RPL, int G>
 __global__ void __launch_bounds__(64)
 gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, int64_t row_stride,
                 const float* __restrict__ alpha, const int* __restrict__ entry_start,
@@ -54,12 +77,17 @@ gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __res
                 float q_scale, float* __restrict__ o) {
     constexpr int STAGE = RPL <= 16 ? 16 : (RPL <= 32 ? 8 : 4);       // tokens staged at a time
     constexpr int ROWS = GLA_GROUPS * RPL;                             // padded rows of a head
-    constexpr int PER_LANE = STAGE * ROWS / 64;                        // staged elements of each array a lane moves
+    constexpr int PIECES = STAGE * ROWS / G / 64;                      // pieces of G rows of each array a lane moves
+    constexpr int VPIECES = (STAGE * GLA_COLS / G + 63) / 64;          // pieces of G columns of v a lane moves
     __shared__ __attribute__((aligned(16))) float sa[STAGE * ROWS];
     __shared__ __attribute__((aligned(16))) float sk[STAGE * ROWS];
     __shared__ __attribute__((aligned(16))) float sq[STAGE * ROWS];
+    __shared__ __attribute__((aligned(16))) float sv[STAGE * GLA_COLS];
+    __shared__ __attribute__((aligned(16))) float so[STAGE * GLA_COLS];
     const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int col = blockIdx.z * GLA_COLS + (lane % GLA_COLS), group = lane / GLA_COLS;
+    const int col0 = blockIdx.z * GLA_COLS;
+    const int colidx = lane / GLA_GROUPS, group = lane % GLA_GROUPS;
+    const int col = col0 + colidx;
     const bool live = col < vdim;
     const int t0 = entry_start[e], t1 = entry_start[e + 1];
     float* S = state + (((int64_t)state_slots[e] * heads + h) * dim) * (int64_t)vdim;
@@ -69,61 +97,101 @@ gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __res
         const int d = group * RPL + i;
         s[i] = (live && d < dim) ? S[(int64_t)d * vdim + col] : 0.f;
     }
-    float na[PER_LANE], nk[PER_LANE], nq[PER_LANE], nv[STAGE];        // the next tokens, on their way from memory
+    GlaRaw<float, G> ra[PIECES];
+    GlaRaw<T, G> rk[PIECES], rq[PIECES], rv[VPIECES];
 
+    // piece p of a stage's rows: token p / (ROWS / G) of the stage, rows G * (p % (ROWS / G)) ..; where that lies past
+    // the entry's tokens or the head's rows, a piece that exists is read instead and is not used
     auto fetch = [&](int base) {
 #pragma unroll
-        for (int j = 0; j < PER_LANE; ++j) {
-            const int el = lane + 64 * j, tt = el / ROWS, d = el % ROWS, t = base + tt;
-            const bool there = t < t1 && d < dim;
+        for (int j = 0; j < PIECES; ++j) {
+            const int piece = lane + 64 * j;
+            const int t = min(base + piece / (ROWS / G), t1 - 1), d = min(G * (piece % (ROWS / G)), dim - G);
             const int64_t at = (int64_t)t * row_stride + (int64_t)h * dim + d;
-            na[j] = there ? alpha[((int64_t)t * heads + h) * dim + d] : 0.f;
-            nk[j] = there ? to_float(k[at]) : 0.f;
-            nq[j] = there ? to_float(q[at]) * q_scale : 0.f;
+            ra[j] = gla_load<float, G>(alpha + ((int64_t)t * heads + h) * dim + d);
+            rk[j] = gla_load<T, G>(k + at);
+            rq[j] = gla_load<T, G>(q + at);
         }
 #pragma unroll
-        for (int tt = 0; tt < STAGE; ++tt)
-            nv[tt] = (live && base + tt < t1) ? to_float(v[(int64_t)(base + tt) * row_stride + (int64_t)h * vdim + col]) : 0.f;
+        for (int j = 0; j < VPIECES; ++j) {
+            const int piece = lane + 64 * j;
+            const int t = min(base + piece / (GLA_COLS / G), t1 - 1);
+            const int c = min(col0 + G * (piece % (GLA_COLS / G)), vdim - G);
+            rv[j] = gla_load<T, G>(v + (int64_t)t * row_stride + (int64_t)h * vdim + c);
+        }
     };
 
     if (t0 < t1) fetch(t0);
     for (int base = t0; base < t1; base += STAGE) {
         const int count = min(STAGE, t1 - base);
-        float vt[STAGE];
+        // into LDS, converted: a row past dim keeps its zero; a token past the entry's last leaves the state as it is
+        // (alpha 1, k 0)
 #pragma unroll
-        for (int j = 0; j < PER_LANE; ++j) {
-            sa[lane + 64 * j] = na[j];
-            sk[lane + 64 * j] = nk[j];
-            sq[lane + 64 * j] = nq[j];
-        }
+        for (int j = 0; j < PIECES; ++j) {
+            const int piece = lane + 64 * j;
+            const int tt = piece / (ROWS / G), d = G * (piece % (ROWS / G));
+            const bool token_there = base + tt < t1;
 #pragma unroll
-        for (int tt = 0; tt < STAGE; ++tt) vt[tt] = nv[tt];
-        __syncthreads();                           // one wavefront a workgroup: its stores to LDS before its reads
-        if (base + STAGE < t1) fetch(base + STAGE);
-#pragma unroll
-        for (int tt = 0; tt < STAGE; ++tt) {
-            if (tt < count) {
-                const float* a = sa + tt * ROWS + group * RPL;
-                const float* kk = sk + tt * ROWS + group * RPL;
-                const float* qq = sq + tt * ROWS + group * RPL;
-                float acc = 0.f;
-#pragma unroll
-                for (int i = 0; i < RPL; i += 4) {
-                    const gla_f32x4 a4 = *reinterpret_cast<const gla_f32x4*>(a + i);
-                    const gla_f32x4 k4 = *reinterpret_cast<const gla_f32x4*>(kk + i);
-                    const gla_f32x4 q4 = *reinterpret_cast<const gla_f32x4*>(qq + i);
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        s[i + x] = fmaf(a4[x], s[i + x], k4[x] * vt[tt]);
-                        acc = fmaf(s[i + x], q4[x], acc);
-                    }
-                }
-                acc += __shfl_xor(acc, GLA_COLS, 64);
-                acc += __shfl_xor(acc, 2 * GLA_COLS, 64);
-                if (live && group == 0) o[((int64_t)(base + tt) * heads + h) * vdim + col] = acc;
+            for (int x = 0; x < G; ++x) {
+                const bool row_there = d + x < dim;          // with G == 4 a piece is there whole or not at all
+                const bool there = token_there && row_there;
+                sa[piece * G + x] = there ? ra[j].v[x] : (row_there ? 1.f : 0.f);
+                sk[piece * G + x] = there ? to_float(rk[j].v[x]) : 0.f;
+                sq[piece * G + x] = there ? to_float(rq[j].v[x]) * q_scale : 0.f;
             }
         }
-        __syncthreads();                           // the reads, before the next tokens are staged
+#pragma unroll
+        for (int j = 0; j < VPIECES; ++j) {
+            const int piece = lane + 64 * j;
+            if (piece < STAGE * GLA_COLS / G) {
+                const int tt = piece / (GLA_COLS / G), c = G * (piece % (GLA_COLS / G));
+#pragma unroll
+                for (int x = 0; x < G; ++x)
+                    sv[piece * G + x] = (base + tt < t1 && col0 + c + x < vdim) ? to_float(rv[j].v[x]) : 0.f;
+            }
+        }
+        __syncthreads();                           // one wavefront a workgroup: its stores to LDS before its reads
+        if (base + STAGE < t1) fetch(base + STAGE);
+        // every staged token is worked on, also those past the entry's last (they change nothing and store nothing), so
+        // that the tokens' instructions can be woven into each other
+#pragma unroll
+        for (int tt = 0; tt < STAGE; ++tt) {
+            const float* a = sa + tt * ROWS + group * RPL;
+            const float* kk = sk + tt * ROWS + group * RPL;
+            const float* qq = sq + tt * ROWS + group * RPL;
+            const float vt = sv[tt * GLA_COLS + colidx];
+            float part[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < RPL; i += 4) {
+                const gla_f32x4 a4 = *reinterpret_cast<const gla_f32x4*>(a + i);
+                const gla_f32x4 k4 = *reinterpret_cast<const gla_f32x4*>(kk + i);
+                const gla_f32x4 q4 = *reinterpret_cast<const gla_f32x4*>(qq + i);
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    s[i + x] = fmaf(a4[x], s[i + x], k4[x] * vt);
+                    part[x] = fmaf(s[i + x], q4[x], part[x]);
+                }
+            }
+            float acc = (part[0] + part[1]) + (part[2] + part[3]);
+            acc += quad_swap<0xB1>(acc);           // the neighbour in the quad, then the other pair: the four row groups
+            acc += quad_swap<0x4E>(acc);
+            if (group == 0) so[tt * GLA_COLS + colidx] = acc;
+        }
+        __syncthreads();                           // the reads, before the next tokens are staged; so is whole
+        // the stage's o: token lane / 4, columns 4 * (lane % 4) .. + 3
+        if (lane < STAGE * 4) {
+            const int tt = lane / 4, c = 4 * (lane % 4);
+            if (tt < count) {
+                float* row = o + ((int64_t)(base + tt) * heads + h) * vdim + col0 + c;
+                if (G == 4) {
+                    if (col0 + c < vdim) *reinterpret_cast<gla_f32x4*>(row) = *reinterpret_cast<const gla_f32x4*>(so + tt * GLA_COLS + c);
+                } else {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x)
+                        if (col0 + c + x < vdim) row[x] = so[tt * GLA_COLS + c + x];
+                }
+            }
+        }
     }
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
@@ -147,9 +215,21 @@ extern "C" int somi_gla_scan(const void* q, const void* k, const void* v, int dt
     if (n_entries == 0) return 0;
     const dim3 grid(n_entries, heads, ceil_div(vdim, GLA_COLS));
     const int rpl = ceil_div(dim, GLA_GROUPS);
+    // four elements at a time where every piece of four is whole and aligned
+    const bool wide = dim % 4 == 0 && vdim % 4 == 0 && row_stride % 4 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)k % 8 == 0 &&
+                      (uintptr_t)v % 8 == 0 && (uintptr_t)alpha % 16 == 0 && (uintptr_t)o % 16 == 0 &&
+                      (dtype == SOMI_BF16 || ((uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0));
 #define GLA_LAUNCH(T, R)                                                                                              \
-    hipLaunchKernelGGL((gla_scan_kernel<T, R>), grid, dim3(64), 0, stream, (const T*)q, (const T*)k, (const T*)v,     \
-                       row_stride, alpha, entry_start, state_slots, state, heads, dim, vdim, q_scale, o)
+    do {                                                                                                              \
+        if (wide)                                                                                                     \
+            hipLaunchKernelGGL((gla_scan_kernel<T, R, 4>), grid, dim3(64), 0, stream, (const T*)q, (const T*)k,       \
+                               (const T*)v, row_stride, alpha, entry_start, state_slots, state, heads, dim, vdim,     \
+                               q_scale, o);                                                                           \
+        else                                                                                                          \
+            hipLaunchKernelGGL((gla_scan_kernel<T, R, 1>), grid, dim3(64), 0, stream, (const T*)q, (const T*)k,       \
+                               (const T*)v, row_stride, alpha, entry_start, state_slots, state, heads, dim, vdim,     \
+                               q_scale, o);                                                                           \
+    } while (0)
 #define GLA_BY_ROWS(T)                                                                                                \
     do {                                                                                                              \
         if (rpl <= 4) GLA_LAUNCH(T, 4);                                                                               \
