@@ -8,10 +8,13 @@
 // that divides heads / kv_heads) of 16 / HT consecutive tokens of one portion, or of one listed token.  Its four
 // wavefronts take the tile's 16-key tiles in turn (the kept first tokens below the window, then the window; tiles are
 // aligned to absolute positions) and are merged through LDS.  Per key tile and map, in a wavefront:
-//   S^T[key, slot] = K[key, :] . Q^T      v_mfma_f32_16x16x16_bf16; K rows are the A operand.  The sum over the key
+//   S^T[key, slot] = K[key, :] . Q^T      v_mfma_f32_16x16x16_bf16 (16x16x32 where a quarter of a key row is a multiple
+//                                         of eight channels); K rows are the A operand.  The sum over the key
 //                                         channels has no order, so lane group g takes the g-th quarter of a row:
 //                                         one contiguous read of dk / 4 channels per lane
-//   mask by the slot's own position, online softmax per slot in float32 (a lane holds four keys of its slot)
+//   mask by the slot's own position (tiles that every slot sees whole skip it), online softmax per slot in float32
+//                                         in powers of two (a lane holds four keys of its slot) against a reference
+//                                         point that follows the slot's maximum lazily
 //   O^T[channel, slot] += V^T[channel, key] . P^T     S^T leaves the first product in the B-operand layout of the
 //                                         second, and V is stored transposed inside a page, so a lane reads four
 //                                         consecutive keys of a channel with one 8-byte load, once for both maps.
@@ -23,8 +26,10 @@
 typedef __attribute__((ext_vector_type(4))) __bf16 dmf_bf16x4;
 typedef __attribute__((ext_vector_type(4))) short dmf_short4;
 typedef __attribute__((ext_vector_type(4))) float dmf_f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 dmf_bf16x8;
 
 #define DMF_WAVES 4
+#define DMF_SLACK 8.0f            // powers of two a score may pass its slot's reference point by before the point moves
 
 struct DiffArgs {
     const bf16* q; int64_t q_stride;
@@ -40,6 +45,7 @@ struct DiffArgs {
 };
 
 __device__ __forceinline__ dmf_short4 dmf_ld4(const bf16* p) { return *reinterpret_cast<const dmf_short4*>(p); }
+__device__ __forceinline__ dmf_bf16x8 dmf_ld8(const bf16* p) { return *reinterpret_cast<const dmf_bf16x8*>(p); }
 
 template <int DKT, int DVT>
 __global__ void __launch_bounds__(DMF_WAVES * 64)
@@ -78,17 +84,27 @@ diff_attention_mfma_kernel(const DiffArgs a) {
     const int pq = live ? p0 + slot_token : -1;                    // the slot's position; -1 sees nothing
     const int* table = a.block_table + (int64_t)e * a.max_blocks;
 
-    // ---- the slot's two queries: lane group g holds channels g * DK/4 .. + DK/4 - 1, four per product step
-    dmf_short4 qf[2][DKT];
+    // ---- the slot's two queries: lane group g holds channels g * DK/4 .. + DK/4 - 1; a product step takes four of
+    // them (v_mfma_f32_16x16x16_bf16), or eight where a quarter of a row is a multiple of eight
+    // (v_mfma_f32_16x16x32_bf16: half the instructions, 16-byte reads)
+    constexpr bool WIDE = DKT % 2 == 0;
+    constexpr int QSTEPS = WIDE ? DKT / 2 : DKT;
+    dmf_short4 qf[2][WIDE ? 1 : DKT];
+    dmf_bf16x8 qw[2][WIDE ? QSTEPS : 1];
 #pragma unroll
-    for (int map = 0; map < 2; ++map)
+    for (int map = 0; map < 2; ++map) {
+        const bf16* qrow = a.q + (int64_t)(t0 + (live ? slot_token : 0)) * a.q_stride + (int64_t)(2 * head + map) * DK + g * (DK / 4);
 #pragma unroll
-        for (int kk = 0; kk < DKT; ++kk) {
-            qf[map][kk] = dmf_short4{0, 0, 0, 0};
-            if (live)
-                qf[map][kk] = dmf_ld4(a.q + (int64_t)(t0 + slot_token) * a.q_stride + (int64_t)(2 * head + map) * DK +
-                                      g * (DK / 4) + 4 * kk);
+        for (int kk = 0; kk < QSTEPS; ++kk) {
+            if (WIDE) {
+                qw[map][kk] = dmf_bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (live) qw[map][kk] = dmf_ld8(qrow + 8 * kk);
+            } else {
+                qf[map][kk] = dmf_short4{0, 0, 0, 0};
+                if (live) qf[map][kk] = dmf_ld4(qrow + 4 * kk);
+            }
         }
+    }
 
     // ---- the key tiles of the query tile: kept first tokens below its window, then the window
     const int pmin = p0, pmax = p0 + count - 1;
@@ -107,6 +123,7 @@ diff_attention_mfma_kernel(const DiffArgs a) {
         for (int c = 0; c < DVT; ++c) acc[map][c] = dmf_f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int last_block = a.max_blocks - 1;
+    const float scale2 = a.scale * 1.4426950408889634f;            // scores in units of log 2
     for (int idx = wave; idx < tiles; idx += DMF_WAVES) {
         const int tile = idx < sink_tiles ? idx : w0 + (idx - sink_tiles);
         const int j0 = tile << 4;
@@ -119,57 +136,94 @@ diff_attention_mfma_kernel(const DiffArgs a) {
         const int vpos = min(j0 + 4 * g, pmax & ~3);
         const int64_t vpage = table[min(vpos / a.page_size, last_block)];
         const bf16* vbase = a.vc + (vpage * a.nkv + kvh) * (int64_t)DV * a.page_size + vpos % a.page_size;
-        dmf_short4 kf[2][DKT], vf[DVT];
+        dmf_short4 kf[2][WIDE ? 1 : DKT], vf[DVT];
+        dmf_bf16x8 kw[2][WIDE ? QSTEPS : 1];
 #pragma unroll
         for (int map = 0; map < 2; ++map)
 #pragma unroll
-            for (int kk = 0; kk < DKT; ++kk) kf[map][kk] = dmf_ld4(krow + (int64_t)map * a.page_size * DK + 4 * kk);
+            for (int kk = 0; kk < QSTEPS; ++kk) {
+                if (WIDE) kw[map][kk] = dmf_ld8(krow + (int64_t)map * a.page_size * DK + 8 * kk);
+                else kf[map][kk] = dmf_ld4(krow + (int64_t)map * a.page_size * DK + 4 * kk);
+            }
 #pragma unroll
         for (int c = 0; c < DVT; ++c) vf[c] = dmf_ld4(vbase + (int64_t)(c * 16 + r) * a.page_size);
-        // a key that no slot of the tile sees (past the last written position, or below the window in a page that
-        // was given back) may hold anything: its weight is 0, but 0 x NaN is NaN
+        // A tile whose every key every slot of the query tile sees (it ends at or before the first slot's position,
+        // and begins inside the last slot's window or lies among the kept tokens) needs no mask: most tiles of a
+        // long window.
+        const bool full = j0 + 15 <= pmin && (a.window == 0 || pmax - j0 < a.window || j0 + 15 < a.keep_first);
+        if (!full) {
+            // a key that no slot of the tile sees (past the last written position, or below the window in a page that
+            // was given back) may hold anything: its weight is 0, but 0 x NaN is NaN
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int j = j0 + 4 * g + i;
-            if (j > pmax || (j < wlo && j >= a.keep_first)) {
+            for (int i = 0; i < 4; ++i) {
+                const int j = j0 + 4 * g + i;
+                if (j > pmax || (j < wlo && j >= a.keep_first)) {
 #pragma unroll
-                for (int c = 0; c < DVT; ++c) vf[c][i] = 0;
+                    for (int c = 0; c < DVT; ++c) vf[c][i] = 0;
+                }
             }
         }
 
         dmf_short4 p_hi[2], p_lo[2];
-        float corr[2];
+        dmf_f32x4 s[2];
+        float mx[2];
 #pragma unroll
         for (int map = 0; map < 2; ++map) {
-            dmf_f32x4 s = {0.f, 0.f, 0.f, 0.f};
+            s[map] = dmf_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kk = 0; kk < DKT; ++kk)
-                s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf[map][kk], qf[map][kk], s, 0, 0, 0);
-            // s[i] = S[key j0 + 4 g + i][slot r]
-            float mx = -INFINITY;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int j = j0 + 4 * g + i;
-                const bool sees = j <= pq && (a.window == 0 || pq - j < a.window || j < a.keep_first);
-                s[i] = sees ? s[i] * a.scale : -INFINITY;
-                mx = fmaxf(mx, s[i]);
+            for (int kk = 0; kk < QSTEPS; ++kk) {
+                if (WIDE) s[map] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kw[map][kk], qw[map][kk], s[map], 0, 0, 0);
+                else s[map] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf[map][kk], qf[map][kk], s[map], 0, 0, 0);
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m_run[map], mx);
-            const float m_safe = m_new == -INFINITY ? 0.f : m_new;      // a slot that has seen no key yet
-            corr[map] = expf(m_run[map] - m_safe);
+            // s[i] = S[key j0 + 4 g + i][slot r], from here on in units of log 2: the weights are powers of two
+            mx[map] = -INFINITY;
+            if (full) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    s[map][i] *= scale2;
+                    mx[map] = fmaxf(mx[map], s[map][i]);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int j = j0 + 4 * g + i;
+                    const bool sees = j <= pq && (a.window == 0 || pq - j < a.window || j < a.keep_first);
+                    s[map][i] = sees ? s[map][i] * scale2 : -INFINITY;
+                    mx[map] = fmaxf(mx[map], s[map][i]);
+                }
+            }
+        }
+        // The weights are taken against a reference point per slot and map that follows the maximum lazily: it moves
+        // (and the sums so far are rescaled) only when a score passes it by more than DMF_SLACK powers of two, which
+        // the whole wavefront decides together; until then no lane looks at another lane's scores.
+        if (__any(mx[0] > m_run[0] + DMF_SLACK || mx[1] > m_run[1] + DMF_SLACK)) {
+#pragma unroll
+            for (int map = 0; map < 2; ++map) {
+                float top = mx[map];
+                top = fmaxf(top, __shfl_xor(top, 16, 64));
+                top = fmaxf(top, __shfl_xor(top, 32, 64));
+                if (top > m_run[map] + DMF_SLACK) {                   // the slot's four lanes agree: top is theirs together
+                    const float corr = m_run[map] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[map] - top);
+                    l_run[map] *= corr;
+#pragma unroll
+                    for (int c = 0; c < DVT; ++c) acc[map][c] *= corr;
+                    m_run[map] = top;
+                }
+            }
+        }
+#pragma unroll
+        for (int map = 0; map < 2; ++map) {
+            const float m_safe = m_run[map] == -INFINITY ? 0.f : m_run[map];      // a slot that has seen no key yet
             float sum = 0.f;
             dmf_bf16x4 hi, lo;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float p = expf(s[i] - m_safe);
+                const float p = __builtin_amdgcn_exp2f(s[map][i] - m_safe);
                 sum += p;
                 hi[i] = (bf16)p;
                 lo[i] = (bf16)(p - (float)hi[i]);
             }
-            l_run[map] = l_run[map] * corr[map] + sum;                  // the lane's own keys; lane groups are added at the end
-            m_run[map] = m_new;
+            l_run[map] += sum;                                          // the lane's own keys; lane groups are added at the end
             p_hi[map] = *reinterpret_cast<dmf_short4*>(&hi);
             p_lo[map] = *reinterpret_cast<dmf_short4*>(&lo);
         }
@@ -177,7 +231,6 @@ diff_attention_mfma_kernel(const DiffArgs a) {
         for (int map = 0; map < 2; ++map)
 #pragma unroll
             for (int c = 0; c < DVT; ++c) {
-                acc[map][c] *= corr[map];
                 acc[map][c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[c], p_hi[map], acc[map][c], 0, 0, 0);
                 acc[map][c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[c], p_lo[map], acc[map][c], 0, 0, 0);
             }
@@ -210,7 +263,7 @@ diff_attention_mfma_kernel(const DiffArgs a) {
 #pragma unroll
         for (int w = 0; w < DMF_WAVES; ++w) {
             const float mw = lds_m[(w * 2 + map) * 16 + r];
-            factor[map][w] = (m_all > -INFINITY && mw > -INFINITY) ? expf(mw - m_all) : 0.f;
+            factor[map][w] = (m_all > -INFINITY && mw > -INFINITY) ? exp2f(mw - m_all) : 0.f;
             l_all[map] += lds_l[(w * 2 + map) * 16 + r] * factor[map][w];
         }
     }
@@ -316,6 +369,9 @@ extern "C" int somi_diff_attention_mfma(const void* q, int64_t q_stride, const v
     SOMI_REQUIRE(window >= 0 && keep_first >= 0, "diff_attention_mfma: window and keep_first must be >= 0");
     SOMI_REQUIRE(q_stride % 4 == 0 && (uintptr_t)q % 8 == 0 && (uintptr_t)k_cache % 8 == 0 && (uintptr_t)v_cache % 8 == 0 &&
                  (uintptr_t)out % 8 == 0, "diff_attention_mfma: operands must be aligned to 8 bytes");
+    // key sizes of a multiple of 32 read a quarter of a row sixteen bytes at a time
+    SOMI_REQUIRE(dk % 32 != 0 || (q_stride % 8 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)k_cache % 16 == 0),
+                 "diff_attention_mfma: with a key size of %d the queries and the key cache must be aligned to 16 bytes", dk);
     DiffArgs args;
     args.q = (const bf16*)q; args.q_stride = q_stride; args.kc = (const bf16*)k_cache; args.vc = (const bf16*)v_cache;
     args.block_table = block_table; args.max_blocks = max_blocks;

@@ -853,7 +853,8 @@ def gla_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, eps
 def diff_attention_mfma_supported(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> bool:
     """The matrix-core kernel takes these operands: bfloat16, key and value sizes it is built for, pages of a multiple
     of 4 keys, rows aligned to 8 bytes."""
-    return (q.dtype == torch.bfloat16 and q.shape[1] % 4 == 0 and q.data_ptr() % 8 == 0
+    wide = k_cache.shape[3] % 32 == 0          # such key sizes are read sixteen bytes at a time
+    return (q.dtype == torch.bfloat16 and q.shape[1] % (8 if wide else 4) == 0 and q.data_ptr() % (16 if wide else 8) == 0
             and bool(library().somi_diff_attention_mfma_supported(k_cache.shape[3], v_cache.shape[2], k_cache.shape[2])))
 
 
