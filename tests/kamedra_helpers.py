@@ -24,6 +24,8 @@ def attention(heads, kv_heads, dim, vdim, size, keep_first, rot_dims, base=10000
 #    rescaling; a window longer than any test sequence; more kept tokens than the window is long; one recurrent head;
 #    tau = 1; no soft cap; attention first.
 # C: large recurrent heads; attention without rotation and a window of a few tokens; lender and borrower alike.
+# D: recurrent layers only (no paged cache at all), a width that is no multiple of 32.
+# E: attention layers only (no state), one head, a lender with two borrowers of different masks, a window of one token.
 KAMEDRA = {
     "A": dict(block_size=16, seed=5, config=KamedraConfig(vocab=211, width=96, norm_eps=1e-5, logit_softcap=20.0, layers=(
         KamedraLayer("gla", KamedraGLA(heads=3, dim=16, vdim=32, tau=8.0, rank=8)),
@@ -40,6 +42,15 @@ KAMEDRA = {
         KamedraLayer("gla", KamedraGLA(heads=2, dim=64, vdim=128, tau=32.0, rank=16), ff=96),
         KamedraLayer("attention", attention(2, 2, 48, 32, 16, 1, 0, diff=0.5, scale=0.15)),
         KamedraLayer("attention", attention(2, 2, 48, 32, 16, 1, 0, diff=0.5, scale=0.15, kv_from=1), ff=48),
+    ))),
+    "D": dict(block_size=16, seed=8, config=KamedraConfig(vocab=61, width=48, norm_eps=1e-6, logit_softcap=15.0, layers=(
+        KamedraLayer("gla", KamedraGLA(heads=2, dim=12, vdim=20, tau=4.0, rank=6), ff=72),
+        KamedraLayer("gla", KamedraGLA(heads=4, dim=8, vdim=16, tau=2.0, rank=3)),
+    ))),
+    "E": dict(block_size=8, seed=9, config=KamedraConfig(vocab=83, width=64, norm_eps=1e-5, logit_softcap=None, layers=(
+        KamedraLayer("attention", attention(1, 1, 32, 32, 12, 2, 32, base=100.0, diff=0.3, scale=0.2)),
+        KamedraLayer("attention", attention(1, 1, 32, 32, 1, 0, 32, base=100.0, diff=0.8, scale=0.3, kv_from=0), ff=40),
+        KamedraLayer("attention", attention(1, 1, 32, 32, 50, 7, 32, base=100.0, diff=0.2, scale=0.1, kv_from=0)),
     ))),
 }
 
