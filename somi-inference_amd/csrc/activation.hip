@@ -71,8 +71,9 @@ extern "C" int somi_silu_mul(const void* gate_up, void* out, int dtype, int n_to
     return 0;
 }
 
-// The gated product with a choice of activation: out[t, i] = act(gate[t, i]) * up[t, i], gu = [gate columns | up
-// columns].  act 0: SiLU; act 1: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+// The gated product with a choice of activation: out[t, i] = act(gate[t, i]) * up[t, i]; gu = [gate columns | up
+// columns] (block == 0) or gate and up columns interleaved in blocks of `block` columns, as for somi_silu_mul.
+// act 0: SiLU; act 1: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
 __device__ __forceinline__ float gelu_tanh(float z) {
     const float inner = 0.7978845608028654f * (z + 0.044715f * z * z * z);
     return 0.5f * z * (1.0f + tanhf(inner));
@@ -80,30 +81,33 @@ __device__ __forceinline__ float gelu_tanh(float z) {
 
 template <typename T>
 __global__ void __launch_bounds__(256)
-act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int act, int64_t count) {
+act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int act, int block, int64_t count) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256) {
         const int64_t t = i / inter;
         const int c = (int)(i - t * inter);
-        const float g = to_float(gu[t * 2 * inter + c]);
-        const float u = to_float(gu[t * 2 * inter + inter + c]);
+        const int at_gate = block > 0 ? (c / block) * 2 * block + c % block : c;
+        const int at_up = block > 0 ? at_gate + block : inter + c;
+        const float g = to_float(gu[t * 2 * inter + at_gate]);
+        const float u = to_float(gu[t * 2 * inter + at_up]);
         const float a = act == 1 ? gelu_tanh(g) : g / (1.0f + expf(-g));
         out[i] = from_float<T>(a * u);
     }
 }
 
-extern "C" int somi_act_mul(const void* gate_up, void* out, int dtype, int n_tokens, int inter, int act,
+extern "C" int somi_act_mul(const void* gate_up, void* out, int dtype, int n_tokens, int inter, int act, int block,
                             hipStream_t stream) {
     SOMI_REQUIRE(n_tokens >= 0 && inter > 0, "act_mul: bad sizes n=%d inter=%d", n_tokens, inter);
+    SOMI_REQUIRE(block >= 0 && (block == 0 || inter % block == 0), "act_mul: block %d does not divide %d", block, inter);
     SOMI_REQUIRE(act == 0 || act == 1, "act_mul: unknown activation %d", act);
     const int64_t count = (int64_t)n_tokens * inter;
     if (count == 0) return 0;
     const int grid = (int)(ceil_div64(count, 256) < 65536 ? ceil_div64(count, 256) : 65536);
     if (dtype == SOMI_F32)
         hipLaunchKernelGGL(act_mul_kernel<float>, dim3(grid), dim3(256), 0, stream, (const float*)gate_up, (float*)out,
-                           inter, act, count);
+                           inter, act, block, count);
     else if (dtype == SOMI_BF16)
         hipLaunchKernelGGL(act_mul_kernel<bf16>, dim3(grid), dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out,
-                           inter, act, count);
+                           inter, act, block, count);
     else
         return somi_fail("act_mul: unknown dtype %d", dtype);
     SOMI_LAUNCH_CHECK("act_mul");

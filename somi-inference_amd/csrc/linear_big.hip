@@ -102,6 +102,7 @@ struct BigArgs {
     bf16* k_cache;                    // [pages, nkv, page_size, D]
     bf16* v_cache;                    // [pages, nkv, D, page_size]
     int nq, nkv, D, page_size;
+    int act;                          // the gated form's activation: 0 or 1 SiLU, 2 the tanh form of GELU
 };
 
 // silu(gate) * up = gate * up / (1 + e^-gate) with the hardware's base-2 exponential and reciprocal (each within
@@ -113,6 +114,14 @@ __device__ __forceinline__ float big_scale_bias(float scale, float sum, float bi
 
 __device__ __forceinline__ float big_silu_mul(float gate, float up) {
     return gate * up * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504088896341f * gate));
+}
+
+// The gated form's end with a choice of activation.  The tanh form of GELU is gate * sigmoid(2 u) with
+// u = sqrt(2 / pi) (gate + 0.044715 gate^3): the same nine instructions with another exponent.
+__device__ __forceinline__ float big_gated(float gate, float up, int act) {
+    if (act != 2) return big_silu_mul(gate, up);
+    const float arg = -2.302208198f * gate * __builtin_fmaf(0.044715f * gate, gate, 1.0f);      // -2 log2(e) u
+    return gate * up * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(arg));
 }
 
 template <int N> __device__ __forceinline__ void big_wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
@@ -479,7 +488,7 @@ linear_big_kernel(const BigArgs p) {
 #pragma unroll
                             for (int c = 0; c < 4; ++c) {
                                 const float gate = s * t[4 * g + c], up = s * t[4 * g + c + 8];
-                                v[c] = (bf16)big_silu_mul(gate, up);
+                                v[c] = (bf16)big_gated(gate, up, p.act);
                             }
                             *(bf16x4*)(stg + ml * SROW + (j * 16 + 8 * g + 4 * nh) * 2) = v;
                         }
@@ -800,7 +809,7 @@ big_stream_finish_kernel(const BigArgs p, int epi) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const float gate = scale * sum[q][e], u = scale * up[q][e];
-                    v[e] = (bf16)big_silu_mul(gate, u);
+                    v[e] = (bf16)big_gated(gate, u, p.act);
                 }
             } else {
                 gc = gn;
@@ -876,7 +885,7 @@ big_split_reduce_swiglu_kernel(const BigArgs p) {
     const float scale = p.row_scale != nullptr ? p.row_scale[gm] : 1.f;
     bf16x4 v;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] = (bf16)big_silu_mul(scale * gate[e], scale * up[e]);
+    for (int e = 0; e < 4; ++e) v[e] = (bf16)big_gated(scale * gate[e], scale * up[e], p.act);
     const int gc = (gn >> 5) * 16 + (gn & 15);
     bf16* dst = p.out + (int64_t)gm * p.ldo + gc;
     if ((p.ldo & 3) == 0 && ((uintptr_t)p.out & 7) == 0) *(bf16x4*)dst = v;
@@ -1229,7 +1238,7 @@ extern "C" int somi_linear_big_tail(int m, int n, int k, int64_t workspace_float
 }
 
 // out = s * (x . w^T) + bias -> bfloat16 [M, N]; with swiglu w is [N, K] with gate and up rows interleaved in blocks
-// of 16 and out is [M, N / 2] = silu(s g) * (s u).  row_scale (or null): s [M], see somi_row_scale.  workspace (or
+// of 16 and out is [M, N / 2] = act(s g) * (s u), act SiLU (swiglu == 1) or the tanh form of GELU (swiglu == 2).  row_scale (or null): s [M], see somi_row_scale.  workspace (or
 // null): as in somi_linear_big_residual, for the plain form (q/k/v of some hundred rows: 72 tiles at 7B sizes).
 extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_t ldw, const float* bias, void* out,
                                int m, int n, int k, const float* row_scale, int swiglu, int tile, float* workspace,
@@ -1241,6 +1250,7 @@ extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_
     BigArgs args = {};
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
     args.M = m; args.N = n; args.K = k; args.out = (bf16*)out; args.ldo = swiglu ? n / 2 : n;
+    args.act = swiglu;                     // 1: SiLU, 2: the tanh form of GELU
     args.row_scale = row_scale;
     SOMI_REQUIRE(workspace == nullptr || (((uintptr_t)workspace & 15) == 0 && workspace_floats >= 0),
                  "linear_big: the workspace must be aligned to 16 bytes");

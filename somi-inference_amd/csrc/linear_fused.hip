@@ -45,6 +45,7 @@ struct FusedRope {
     bf16* k_cache;            // [pages, nkv, page_size, D]
     bf16* v_cache;            // [pages, nkv, D, page_size]
     int nq, nkv, D, page_size;
+    int act;                  // the gated form's activation: 0 or 1 SiLU, 2 the tanh form of GELU
 };
 
 template <int MT, int NS, int MODE, typename TO, bool SWIGLU, bool TAIL, bool ROPE = false>
@@ -317,7 +318,7 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
                 gate *= row_scale[m];
                 up *= row_scale[m];
             }
-            if (n < n_out && m < M) out[(int64_t)m * n_out + n] = from_float<TO>(gate / (1.0f + expf(-gate)) * up);
+            if (n < n_out && m < M) out[(int64_t)m * n_out + n] = from_float<TO>(somi_gated(gate, up, rope.act));
         }
         return;
     }
@@ -468,7 +469,7 @@ extern "C" int somi_linear_residual(const void* x, const void* w, const float* b
 }
 
 // out = s * (x . w^T) (+ bias) with the row scales s[m] = 1 / sqrt(sum of stats[:, m] / K + eps), or with swiglu
-// (w: [2 I, K], gate and up rows interleaved in blocks of 16, no bias) out[m, i] = silu(s g) * (s u) for the gate
+// (w: [2 I, K], gate and up rows interleaved in blocks of 16, no bias) out[m, i] = act(s g) * (s u) (swiglu 1: SiLU, 2: the tanh form of GELU) for the gate
 // and up products g, u.  x: [M, K] bfloat16, the rows a product into the stream wrote as xnext; stats:
 // [stats_blocks][16 ceil(M / 16)] float32 from the same call; out: bfloat16.  M <= 64.
 extern "C" int somi_linear_scaled(const void* x, float eps, const float* stats, int stats_blocks, const void* w,
@@ -478,8 +479,11 @@ extern "C" int somi_linear_scaled(const void* x, float eps, const float* stats, 
     SOMI_REQUIRE(!swiglu || (N % 32 == 0 && bias == nullptr), "linear_scaled: the gated form needs whole pairs of strips and no bias");
     if (M == 0) return 0;
     const int strips = fused_strips(M, N, swiglu != 0);
-    if (swiglu)
-        return fused_launch<2, FUSED_SCALED, bf16, true>(x, w, bias, out, nullptr, nullptr, eps, stats, stats_blocks, nullptr, nullptr, M, N, K, stream);
+    if (swiglu) {
+        FusedRope options{};
+        options.act = swiglu;                  // 1: SiLU, 2: the tanh form of GELU
+        return fused_launch<2, FUSED_SCALED, bf16, true>(x, w, bias, out, nullptr, nullptr, eps, stats, stats_blocks, nullptr, nullptr, M, N, K, stream, options);
+    }
     if (strips >= 2)
         return fused_launch<2, FUSED_SCALED, bf16, false>(x, w, bias, out, nullptr, nullptr, eps, stats, stats_blocks, nullptr, nullptr, M, N, K, stream);
     return fused_launch<1, FUSED_SCALED, bf16, false>(x, w, bias, out, nullptr, nullptr, eps, stats, stats_blocks, nullptr, nullptr, M, N, K, stream);

@@ -42,6 +42,7 @@ struct MidFusion {
     const float* stats_in;    // scaled: [stats_blocks][16 MT] partial sums of squares of the rows that were normed
     int stats_blocks;
     float eps;
+    int act;                  // the gated form's activation: 0 or 1 SiLU, 2 the tanh form of GELU
 };
 
 // What the end of a fused product reads beside the sums, fetched ahead of its use (in the kernel that adds the
@@ -162,7 +163,7 @@ __device__ __forceinline__ void mid_finish(f32x4 (&acc)[NS][MTH], const MidAhead
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const float gate = acc[2 * p][mt][i] * scale, up = acc[2 * p + 1][mt][i] * scale;
-                    if (n + i < n_out) out[(int64_t)m * n_out + n + i] = from_float<TO>(gate / (1.0f + expf(-gate)) * up);
+                    if (n + i < n_out) out[(int64_t)m * n_out + n + i] = from_float<TO>(somi_gated(gate, up, fusion.act));
                 }
             }
         }
@@ -524,7 +525,9 @@ extern "C" int somi_linear_mid(const void* x, const void* w, const float* bias, 
     if (M == 0) return 0;
     int strips, splits;
     mid_shape(M, N, K, swiglu != 0, workspace ? workspace_floats : 0, somi_units(), &strips, &splits);
-    return mid_dispatch<MID_PLAIN>(x, w, bias, out, out_dtype, M, N, K, strips, splits, swiglu != 0, workspace, MidFusion{}, stream);
+    MidFusion options{};
+    options.act = swiglu;                      // 1: SiLU, 2: the tanh form of GELU
+    return mid_dispatch<MID_PLAIN>(x, w, bias, out, out_dtype, M, N, K, strips, splits, swiglu != 0, workspace, options, stream);
 }
 
 // Column tiles (= rows of the statistics) that somi_linear_mid_residual launches for these sizes.
@@ -575,6 +578,7 @@ extern "C" int somi_linear_mid_scaled(const void* x, float eps, const float* sta
     fusion.stats_in = stats;
     fusion.stats_blocks = stats_blocks;
     fusion.eps = eps;
+    fusion.act = swiglu;                       // 1: SiLU, 2: the tanh form of GELU
     return mid_dispatch<MID_SCALED>(x, w, bias, out, SOMI_BF16, M, N, K, strips, splits, swiglu != 0, workspace, fusion, stream);
 }
 

@@ -31,7 +31,7 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 template <int MT, int NS, int CK, int DEPTH, typename TO, bool SWIGLU, bool TAIL>
 __global__ void __launch_bounds__(SKINNY_MAX_WAVES * 64)
 linear_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const float* __restrict__ bias,
-                     TO* __restrict__ out, int M, int N, int K) {
+                     TO* __restrict__ out, int M, int N, int K, int act) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     constexpr int ROW_BYTES = CK * 2;              // bytes of one row in a chunk: 256 or 128
     constexpr int LPR = ROW_BYTES / 16;            // lanes that read one row: 16 or 8
@@ -182,7 +182,7 @@ linear_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, con
             }
             const int n = n0 / 2 + pair * 16 + (l >> 4) * 4 + i;
             const int m = mt * 16 + (l & 15);
-            if (n < n_out && m < M) out[(int64_t)m * n_out + n] = from_float<TO>(gate / (1.0f + expf(-gate)) * up);
+            if (n < n_out && m < M) out[(int64_t)m * n_out + n] = from_float<TO>(somi_gated(gate, up, act));
         }
         return;
     }
@@ -206,6 +206,10 @@ static size_t skinny_lds(int mt, int strips, int chunk, int waves) {
     return waves * (staging > sums ? staging : sums);
 }
 
+// The activation of the gated form that is being launched (1: SiLU, 2: the tanh form of GELU): set by the entry point,
+// read where the kernel is launched, both in one call on one host thread.
+static thread_local int g_skinny_act = 1;
+
 template <int MT, int NS, int CK, int DEPTH, typename TO, bool SW, bool TL>
 static void skinny_launch_kernel(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                                  int waves, hipStream_t stream) {
@@ -215,7 +219,7 @@ static void skinny_launch_kernel(const void* x, const void* w, const float* bias
         (void)hipFuncSetAttribute((const void*)linear_skinny_kernel<MT, NS, CK, DEPTH, TO, SW, TL>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     hipLaunchKernelGGL((linear_skinny_kernel<MT, NS, CK, DEPTH, TO, SW, TL>), grid, block, smem, stream,
-                       (const bf16*)x, (const bf16*)w, bias, (TO*)out, M, N, K);
+                       (const bf16*)x, (const bf16*)w, bias, (TO*)out, M, N, K, g_skinny_act);
 }
 
 template <int MT, int NS, int CK, int DEPTH, typename TO>
@@ -300,13 +304,23 @@ extern "C" int somi_linear_skinny(const void* x, const void* w, const float* bia
 
 // The gated feed-forward's first product with the gate fused in: w: [2 I, K] holds gate and up rows
 // interleaved in blocks of 16 rows (gate rows 0..15, up rows 0..15, gate rows 16..31, ...); out: [M, I] with
-// out[m, i] = silu(x . gate_i) * (x . up_i).  I must be a multiple of 16.
+// out[m, i] = act(x . gate_i) * (x . up_i), act SiLU (1) or the tanh form of GELU (2).  I must be a multiple of 16.
+extern "C" int somi_linear_skinny_gated(const void* x, const void* w, void* out, int out_dtype, int M, int I, int K,
+                                        int act, hipStream_t stream) {
+    if (skinny_check(x, w, out_dtype, M, 2 * I, K)) return 1;
+    SOMI_REQUIRE(I % 16 == 0, "linear_skinny_gated: the intermediate size %d must be a multiple of 16", I);
+    SOMI_REQUIRE(act == 1 || act == 2, "linear_skinny_gated: activation %d (1: SiLU, 2: the tanh form of GELU)", act);
+    if (M == 0) return 0;
+    g_skinny_act = act;
+    const int rc = skinny_auto(x, w, nullptr, out, out_dtype, M, 2 * I, K, true, stream);
+    g_skinny_act = 1;
+    return rc;
+}
+
+// The same with SiLU: out[m, i] = silu(x . gate_i) * (x . up_i).
 extern "C" int somi_linear_skinny_swiglu(const void* x, const void* w, void* out, int out_dtype, int M, int I, int K,
                                          hipStream_t stream) {
-    if (skinny_check(x, w, out_dtype, M, 2 * I, K)) return 1;
-    SOMI_REQUIRE(I % 16 == 0, "linear_skinny_swiglu: the intermediate size %d must be a multiple of 16", I);
-    if (M == 0) return 0;
-    return skinny_auto(x, w, nullptr, out, out_dtype, M, 2 * I, K, true, stream);
+    return somi_linear_skinny_gated(x, w, out, out_dtype, M, I, K, 1, stream);
 }
 
 // The same product with the launch shape given by the caller (wavefronts per workgroup: 1 to 8; 16-column

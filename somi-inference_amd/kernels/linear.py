@@ -27,15 +27,15 @@ def _mid_is_faster(m: int, n: int, k: int) -> bool:
     return (k >= LONG_K and n <= FEW_COLUMNS_PER_UNIT * units) or n >= MANY_COLUMNS_PER_UNIT * units
 
 
-def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """silu(x @ gate.T) * (x @ up.T) for bfloat16 rows; weight: [2 I, K], gate and up rows interleaved in blocks
-    of 16."""
+def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """act(x @ gate.T) * (x @ up.T) for bfloat16 rows, act "silu" or "gelu_tanh"; weight: [2 I, K], gate and up rows
+    interleaved in blocks of 16."""
     m, k = x.shape
     if m > SKINNY_ROWS:
-        return ops.linear_big(x, weight, swiglu=True)
+        return ops.linear_big(x, weight, swiglu=activation)
     if _mid_is_faster(m, weight.shape[0], k):
-        return ops.linear_mid(x, weight, swiglu=True)
-    return ops.linear_skinny_swiglu(x, weight)
+        return ops.linear_mid(x, weight, swiglu=activation)
+    return ops.linear_skinny_swiglu(x, weight, activation)
 
 
 def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, h: torch.Tensor,
@@ -52,7 +52,7 @@ def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
 
 
 def linear_scaled(x: torch.Tensor, eps: float, stats: torch.Tensor, weight: torch.Tensor,
-                  bias: torch.Tensor | None = None, swiglu: bool = False) -> torch.Tensor:
+                  bias: torch.Tensor | None = None, swiglu: "bool | str" = False) -> torch.Tensor:
     """The product of rows that are still to be normed, by the kernel that :func:`linear` would take for the
     sizes; see :func:`ops.linear_scaled`."""
     if x.shape[0] > ops.FUSED_MAX_ROWS:

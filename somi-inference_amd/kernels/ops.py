@@ -34,6 +34,20 @@ def dtype_code(dtype: torch.dtype) -> int:
     raise KernelError(f"unsupported dtype {dtype}; kernels take float32 and bfloat16")
 
 
+GATED = {"silu": 1, "gelu_tanh": 2}      # the activations the gated products take into their ends
+
+
+def gate_code(swiglu: "bool | str | None") -> int:
+    """0: no gate; 1: SiLU (also for True); 2: the tanh form of GELU."""
+    if not swiglu:
+        return 0
+    if swiglu is True:
+        return 1
+    if swiglu not in GATED:
+        raise KernelError(f"unknown gate activation {swiglu!r}; known: {sorted(GATED)}")
+    return GATED[swiglu]
+
+
 _compute_units: dict[int, int] = {}
 
 
@@ -304,9 +318,9 @@ def silu_mul(gate_up: torch.Tensor, block: int = 0) -> torch.Tensor:
     return out
 
 
-def linear_skinny_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """silu(x @ gate.T) * (x @ up.T) in one kernel for at most 64 bfloat16 rows.  weight: [2 I, K] with
-    gate and up rows interleaved in blocks of 16."""
+def linear_skinny_swiglu(x: torch.Tensor, weight: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """act(x @ gate.T) * (x @ up.T) in one kernel for at most 64 bfloat16 rows, act SiLU or the tanh form of GELU.
+    weight: [2 I, K] with gate and up rows interleaved in blocks of 16."""
     _need(x, "linear input", torch.bfloat16)
     m, k = x.shape
     _need(weight, "gate_up weight", torch.bfloat16)
@@ -314,8 +328,8 @@ def linear_skinny_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         raise KernelError(f"linear_skinny_swiglu: weight {tuple(weight.shape)} does not fit input width {k}")
     inter = weight.shape[0] // 2
     out = torch.empty((m, inter), dtype=x.dtype, device=x.device)
-    _check(library().somi_linear_skinny_swiglu(_ptr(x), _ptr(weight), _ptr(out), dtype_code(x.dtype), m, inter, k,
-                                               _stream()))
+    _check(library().somi_linear_skinny_gated(_ptr(x), _ptr(weight), _ptr(out), dtype_code(x.dtype), m, inter, k,
+                                              gate_code(activation), _stream()))
     return out
 
 
@@ -366,14 +380,14 @@ def big_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def linear_big(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, swiglu: bool = False,
+def linear_big(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, swiglu: "bool | str" = False,
                eps: float = 0.0, stats: torch.Tensor | None = None, tile: int = 0,
                out: torch.Tensor | None = None, split_k: bool = True) -> torch.Tensor:
     """s * (x @ weight.T) (+ bias) -> bfloat16 for any number of rows, on 256-row tiles of the matrix cores.
     With ``stats`` ([blocks, width >= M] partial sums of squares, from :func:`linear_big_residual` or
     :func:`linear_residual`) the rows are scaled by s = 1 / sqrt(stats.sum(0) / K + eps): the product of
     RMS-normed rows when x holds ``norm_weight * h``.  With ``swiglu`` weight is [2 I, K] with gate and up rows
-    interleaved in blocks of 16 and the result is silu(s g) * (s u) -> [M, I].  ``tile``: 0 lets the launcher
+    interleaved in blocks of 16 and the result is act(s g) * (s u) -> [M, I] (True or "silu": SiLU; "gelu_tanh").  ``tile``: 0 lets the launcher
     choose the tile width, 128 or 256 asks for it.  ``split_k``: the ungated form may share a tile's K among
     workgroups (through the device's workspace) where its tiles alone would leave most of the device idle."""
     m, n, k = _big_operands(x, weight, bias, "linear_big")
@@ -393,7 +407,7 @@ def linear_big(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None 
     _need(out, "linear_big out", torch.bfloat16, (m, cols))
     workspace = _mid_workspace(x.device) if split_k else None
     _check(library().somi_linear_big(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(weight), ctypes.c_int64(weight.stride(0)),
-                                     _ptr(bias), _ptr(out), m, n, k, _ptr(row_scale), 1 if swiglu else 0, int(tile),
+                                     _ptr(bias), _ptr(out), m, n, k, _ptr(row_scale), gate_code(swiglu), int(tile),
                                      _ptr(workspace), ctypes.c_int64(workspace.numel() if workspace is not None else 0),
                                      _stream()))
     return out
@@ -540,7 +554,7 @@ def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
 
 
 def linear_scaled(x: torch.Tensor, eps: float, stats: torch.Tensor, weight: torch.Tensor,
-                  bias: torch.Tensor | None = None, swiglu: bool = False, mid: bool = False) -> torch.Tensor:
+                  bias: torch.Tensor | None = None, swiglu: "bool | str" = False, mid: bool = False) -> torch.Tensor:
     """s * (x @ weight.T) (+ bias) -> bfloat16 with the row scales s = 1 / sqrt(stats.sum(0) / K + eps): the
     product of RMS-normed rows when x holds ``norm_weight * h`` and stats the sums of squares of h, both from
     :func:`linear_residual`.  At most 64 rows.  With ``swiglu`` weight is [2 I, K] with gate and up rows
@@ -561,11 +575,11 @@ def linear_scaled(x: torch.Tensor, eps: float, stats: torch.Tensor, weight: torc
     if mid:
         workspace = _mid_workspace(x.device)
         _check(library().somi_linear_mid_scaled(_ptr(x), ctypes.c_float(eps), _ptr(stats), stats.shape[0],
-                                                _ptr(weight), _ptr(bias), _ptr(out), m, n, k, 1 if swiglu else 0,
+                                                _ptr(weight), _ptr(bias), _ptr(out), m, n, k, gate_code(swiglu),
                                                 _ptr(workspace), ctypes.c_int64(workspace.numel()), _stream()))
     else:
         _check(library().somi_linear_scaled(_ptr(x), ctypes.c_float(eps), _ptr(stats), stats.shape[0], _ptr(weight),
-                                            _ptr(bias), _ptr(out), m, n, k, 1 if swiglu else 0, _stream()))
+                                            _ptr(bias), _ptr(out), m, n, k, gate_code(swiglu), _stream()))
     return out
 
 
@@ -611,7 +625,7 @@ def linear_rope_store(x: torch.Tensor, eps: float, stats: torch.Tensor | None, w
 
 
 def linear_mid(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
-               out_dtype: torch.dtype | None = None, swiglu: bool = False) -> torch.Tensor:
+               out_dtype: torch.dtype | None = None, swiglu: "bool | str" = False) -> torch.Tensor:
     """x @ weight.T (+ bias) for at most 64 bfloat16 rows, x shared by the wavefronts of a workgroup, K split
     over workgroups where the columns do not fill the device.  With ``swiglu`` weight is [2 I, K] with gate and
     up rows interleaved in blocks of 16 and the result is silu(x @ gate.T) * (x @ up.T)."""
@@ -627,7 +641,7 @@ def linear_mid(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None 
     out = torch.empty((m, n // 2 if swiglu else n), dtype=out_dtype, device=x.device)
     workspace = _mid_workspace(x.device)
     _check(library().somi_linear_mid(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), dtype_code(out_dtype), m, n, k,
-                                     1 if swiglu else 0, _ptr(workspace), ctypes.c_int64(workspace.numel()), _stream()))
+                                     gate_code(swiglu), _ptr(workspace), ctypes.c_int64(workspace.numel()), _stream()))
     return out
 
 
@@ -713,8 +727,9 @@ def probe_mfma(iters: int, device: torch.device | str = "cuda:0", dense: bool = 
 ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
 
 
-def act_mul(gate_up: torch.Tensor, activation: str) -> torch.Tensor:
-    """act(gate) * up for gate_up = [gate columns | up columns]; ``activation``: one of ACTIVATIONS."""
+def act_mul(gate_up: torch.Tensor, activation: str, block: int = 0) -> torch.Tensor:
+    """act(gate) * up; ``activation``: one of ACTIVATIONS.  block == 0: gate_up = [gate columns | up columns]; block ==
+    b: gate and up columns interleaved in blocks of b columns, as for :func:`silu_mul`."""
     _need(gate_up, "gate_up")
     if activation not in ACTIVATIONS:
         raise KernelError(f"act_mul: unknown activation {activation!r}; known: {sorted(ACTIVATIONS)}")
@@ -723,7 +738,7 @@ def act_mul(gate_up: torch.Tensor, activation: str) -> torch.Tensor:
         raise KernelError(f"act_mul: width {two_i} is odd")
     out = torch.empty((n, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
     _check(library().somi_act_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), n, two_i // 2,
-                                  ACTIVATIONS[activation], _stream()))
+                                  ACTIVATIONS[activation], int(block), _stream()))
     return out
 
 

@@ -13,8 +13,8 @@ from .linear import NormedRows, Projection
 
 
 class SwiGLU(FeedForward):
-    """y = down(act(gate(x)) * up(x)), no biases; ``activation`` is SiLU (the reference's, fused into the gate_up
-    product's end) or the tanh form of GELU (an activation kernel after the product).  gate and up are stacked
+    """y = down(act(gate(x)) * up(x)), no biases; ``activation`` is SiLU (the reference's) or the tanh form of GELU;
+    in bfloat16 either is taken into the gate_up product's end.  gate and up are stacked
     into one ``[2I, H]`` matrix, gate rows first, as the reference merges them at load
     (somi_inference/models/qwen2_adapter.py:183-190, 244-248; qwen2.py:228 chunks the result)."""
     graph_safe = True
@@ -60,7 +60,7 @@ class SwiGLU(FeedForward):
         # (gate 0..15, up 0..15, gate 16..31, ...), so that the decode kernel has gate and up of the same
         # columns in one workgroup and applies the gate in its epilogue.
         self.interleaved = (runtime.dtype == torch.bfloat16 and self.intermediate_size % self.INTERLEAVE == 0
-                            and self.hidden_size % 8 == 0 and self.activation == "silu")
+                            and self.hidden_size % 8 == 0)
         if self.interleaved:
             b, h = self.INTERLEAVE, self.hidden_size
             merged = torch.stack([gate.view(-1, b, h), up.view(-1, b, h)], dim=1).reshape(-1, h).contiguous()
@@ -83,12 +83,15 @@ class SwiGLU(FeedForward):
             if self.gate_up.fusable(x.h.shape[0]):
                 # norm, gate_up and SiLU . up in one kernel
                 with stage(self.gate_up.label):
-                    gated = linear_kernels.linear_scaled(x.weighted, x.norm.eps, x.stats, self.gate_up.weight, swiglu=True)
+                    gated = linear_kernels.linear_scaled(x.weighted, x.norm.eps, x.stats, self.gate_up.weight,
+                                                         swiglu=self.activation)
                 return self.down.deferred(gated)
             x = x.materialize()
         if x.data_ptr() % 16 == 0:
             with stage(self.gate_up.label):
-                return self.down.deferred(linear_kernels.linear_swiglu(x, self.gate_up.weight))
+                return self.down.deferred(linear_kernels.linear_swiglu(x, self.gate_up.weight, self.activation))
         projected = self.gate_up(x)
         with stage("activation"):
-            return self.down.deferred(ops.silu_mul(projected, block=self.INTERLEAVE))
+            if self.activation == "silu":
+                return self.down.deferred(ops.silu_mul(projected, block=self.INTERLEAVE))
+            return self.down.deferred(ops.act_mul(projected, self.activation, block=self.INTERLEAVE))

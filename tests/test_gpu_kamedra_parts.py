@@ -258,9 +258,40 @@ def test_gelu_gate_and_soft_cap(dtype):
     gate_up = rounded(torch.randn(23, 2 * 56) * 3, dtype)
     got = ops.act_mul(gate_up.to(dtype).cuda(), "gelu_tanh").float().cpu()
     torch.testing.assert_close(got, plain.gelu_tanh(gate_up[:, :56]) * gate_up[:, 56:], **tol(dtype))
+    mixed = gate_up.view(23, 2, 7, 8).transpose(1, 2).reshape(23, 112)          # gate and up in blocks of 8 columns
+    again = ops.act_mul(mixed.to(dtype).cuda(), "gelu_tanh", block=8).float().cpu()
+    assert torch.equal(again, got)
     silu = ops.act_mul(gate_up.to(dtype).cuda(), "silu").float().cpu()
     torch.testing.assert_close(silu, torch.nn.functional.silu(gate_up[:, :56]) * gate_up[:, 56:], **tol(dtype))
     logits = torch.randn(7, 301) * 40
     capped = ops.softcap_(logits.clone().cuda(), 30.0).cpu()
     torch.testing.assert_close(capped, 30.0 * torch.tanh(logits / 30.0), rtol=1e-5, atol=1e-5)
     assert float(capped.abs().max()) <= 30.0
+
+
+@pytest.mark.parametrize("rows", [1, 5, 16, 40, 64, 100, 300])
+@pytest.mark.parametrize("inter,hidden", [(64, 96), (160, 64), (2048, 256)])
+def test_gelu_gate_in_the_products_ends(rows, inter, hidden):
+    """The gated feed-forward's first product with the tanh form of GELU taken into its end, by every kernel that the
+    row count and the sizes choose (few rows, split K, many rows; plain and with the norm taken in), against the plain
+    functions."""
+    from somi_inference_amd.kernels import linear as linear_kernels
+    torch.manual_seed(10)
+    x = rounded(torch.randn(rows, hidden), torch.bfloat16)
+    gate = rounded(torch.randn(inter, hidden) * 0.2, torch.bfloat16)
+    up = rounded(torch.randn(inter, hidden) * 0.2, torch.bfloat16)
+    merged = torch.stack([gate.view(-1, 16, hidden), up.view(-1, 16, hidden)], dim=1).reshape(-1, hidden)
+    want = plain.gelu_tanh(x @ gate.t()) * (x @ up.t())
+    got = linear_kernels.linear_swiglu(x.bfloat16().cuda(), merged.bfloat16().cuda(), "gelu_tanh").float().cpu()
+    torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
+    silu = linear_kernels.linear_swiglu(x.bfloat16().cuda(), merged.bfloat16().cuda(), "silu").float().cpu()
+    torch.testing.assert_close(silu, torch.nn.functional.silu(x @ gate.t()) * (x @ up.t()), rtol=2e-2, atol=2e-2)
+    # with the norm taken in: rows h whose weighted copy and sums of squares a product into the stream left
+    h = torch.randn(rows, hidden, device="cuda")
+    weight = (torch.rand(hidden, device="cuda") + 0.5)
+    delta = torch.zeros(rows, 8, device="cuda").bfloat16()
+    stats, weighted = linear_kernels.linear_residual(delta, torch.zeros(hidden, 8, device="cuda").bfloat16(), None, h, weight)
+    # what the product multiplies: the weighted rows as bfloat16 holds them, scaled per row by the norm's factor
+    normed = (weighted.float() / torch.sqrt(h.pow(2).mean(-1, keepdim=True) + 1e-6)).cpu()
+    fused = linear_kernels.linear_scaled(weighted, 1e-6, stats, merged.bfloat16().cuda(), swiglu="gelu_tanh").float().cpu()
+    torch.testing.assert_close(fused, plain.gelu_tanh(normed @ gate.t()) * (normed @ up.t()), rtol=2e-2, atol=2e-2)
