@@ -4,7 +4,8 @@ config.json keys: ``architecture`` ("Kamedra"), ``vocab``, ``width``, ``norm.eps
 list with one object per layer: ``type`` ("attention" or "gla"), ``mixer`` (the mixer's sizes and constants) and
 ``mlp`` (``{"kind": "dense", "ff": ...}`` or null for a layer without a feed-forward).
 
-An attention mixer gives ``heads``, ``kv_heads``, ``dim`` (query/key size of one map), ``vdim``, ``scale``, ``diff``,
+An attention mixer gives ``heads``, ``kv_heads`` (default: ``heads``), ``dim`` (query/key size of one map), ``vdim``
+(default: ``dim``), ``scale`` (default: ``dim^-1/2``), ``diff``,
 ``mask`` (``size``, ``keep_first``), ``rot`` (``base``, ``dims``, optional ``scaling`` with ``factor``, ``low``,
 ``high``, ``original``) and optionally ``kv_from``, the index of the earlier layer whose keys and values it reads.
 A gla mixer gives ``heads``, ``dim``, ``vdim`` and ``tau``; the width of its decay's low-rank projection is the
@@ -52,9 +53,9 @@ class KamedraAttention:
             raise ConfigError(f"{where}: an attention mixer needs 'mask' and 'rot'")
         scaling = rot.sub("scaling")
         out = cls(
-            heads=keys.integer("heads", minimum=1), kv_heads=keys.integer("kv_heads", minimum=1),
-            dim=keys.integer("dim", minimum=1), vdim=keys.integer("vdim", minimum=1),
-            scale=keys.number("scale"), diff=keys.number("diff"),
+            heads=keys.integer("heads", minimum=1), kv_heads=keys.integer("kv_heads", keys.integer("heads", minimum=1), minimum=1),
+            dim=keys.integer("dim", minimum=1), vdim=keys.integer("vdim", keys.integer("dim", minimum=1), minimum=1),
+            scale=keys.number("scale", keys.integer("dim", minimum=1) ** -0.5), diff=keys.number("diff"),
             mask_size=mask.integer("size", minimum=1), mask_keep_first=mask.integer("keep_first", 0, minimum=0),
             rot_base=rot.number("base", positive=True), rot_dims=rot.integer("dims", minimum=0),
             rot_scaling=None if scaling is None else RotaryScaling(
