@@ -1,6 +1,6 @@
 // Differential attention over cache pages on the matrix cores, bfloat16: prompt portions and decoded tokens.
 //
-// The contract of diff_attention.hip (two softmax maps per head over shared values, o = a1 - lambda a2, o divided by
+// What diff_attention.hip computes (two softmax maps per head over shared values, o = a1 - lambda a2, o divided by
 // its root mean square over the head's value channels, times out_scale; a token sees the keys within `window`
 // positions and the first `keep_first` of its request), for key sizes and value sizes that are multiples of 16.
 //
