@@ -187,3 +187,18 @@ def test_greedy_generation_through_the_entry_point(name, dtype, folders):
                 assert gap < (1e-4 if dtype == "float32" else 0.05), f"token {token} instead of {best} (gap {gap})"
             sequence.append(token)
     llm.runner.cache.check_invariants()
+
+
+def test_a_preempted_request_is_recomputed_from_an_empty_state(folders):
+    """A pool too small for three requests: one is preempted, gives back its pages and its state slot, and is run
+    again from its first token later; its recurrent state must start from zero again.  float32: the same tokens."""
+    from somi_inference_amd import LLM
+    prompts = [token_ids(vocab_of("A"), n, 30 + n) for n in (30, 28, 25)]
+    roomy = LLM(folders[("peaky", "A")], dtype="float32", block_size=16, num_blocks=32, max_concurrent=3, eos_token_id=-1)
+    want = roomy.generate(prompts, max_new_tokens=24, temperature=0.0)
+    tight = LLM(folders[("peaky", "A")], dtype="float32", block_size=16, num_blocks=7, max_concurrent=3, eos_token_id=-1)
+    got = tight.generate(prompts, max_new_tokens=24, temperature=0.0)
+    assert tight.scheduler.preemptions > 0 and roomy.scheduler.preemptions == 0
+    assert got == want
+    tight.kv_manager.check_invariants()
+    assert tight.kv_manager.free_pages() == [7]
