@@ -6,7 +6,7 @@
 //
 // A workgroup serves one query tile: 16 (token, head) slots that share a key/value head, HT heads (a power of two
 // that divides heads / kv_heads) of 16 / HT consecutive tokens of one portion, or of one listed token.  Its four
-// wavefronts take the tile's 16-key tiles in turn (the kept first tokens below the window, then the window; tiles are
+// wavefronts (eight for a listed token) take the tile's 16-key tiles in turn (the kept first tokens below the window, then the window; tiles are
 // aligned to absolute positions) and are merged through LDS.  Per key tile and map, in a wavefront:
 //   S^T[key, slot] = K[key, :] . Q^T      v_mfma_f32_16x16x16_bf16 (16x16x32 where a quarter of a key row is a multiple
 //                                         of eight channels); K rows are the A operand.  The sum over the key
@@ -28,7 +28,8 @@ typedef __attribute__((ext_vector_type(4))) short dmf_short4;
 typedef __attribute__((ext_vector_type(4))) float dmf_f32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 dmf_bf16x8;
 
-#define DMF_WAVES 4
+#define DMF_WAVES 4               // wavefronts of a workgroup for portions of prompts
+#define DMF_LISTED_WAVES 8        // and for listed tokens
 #define DMF_SLACK 8.0f            // powers of two a score may pass its slot's reference point by before the point moves
 
 struct DiffArgs {
@@ -47,15 +48,17 @@ struct DiffArgs {
 __device__ __forceinline__ dmf_short4 dmf_ld4(const bf16* p) { return *reinterpret_cast<const dmf_short4*>(p); }
 __device__ __forceinline__ dmf_bf16x8 dmf_ld8(const bf16* p) { return *reinterpret_cast<const dmf_bf16x8*>(p); }
 
-template <int DKT, int DVT>
-__global__ void __launch_bounds__(DMF_WAVES * 64)
+// WAVES: wavefronts of a workgroup, which take the query tile's key tiles in turn: four for portions of prompts (two
+// workgroups fit a compute unit), eight for listed tokens (decoding), whose few query tiles each walk a whole window.
+template <int DKT, int DVT, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
 diff_attention_mfma_kernel(const DiffArgs a) {
     constexpr int DK = 16 * DKT, DV = 16 * DVT;
     extern __shared__ float lds[];
     float* lds_acc = lds;                                          // [waves][2][DVT][64][4]
-    float* lds_m = lds_acc + DMF_WAVES * 2 * DVT * 256;            // [waves][2][16]
-    float* lds_l = lds_m + DMF_WAVES * 32;                         // [waves][2][16]
-    float* lds_ss = lds_l + DMF_WAVES * 32;                        // [waves][16]
+    float* lds_m = lds_acc + WAVES * 2 * DVT * 256;            // [waves][2][16]
+    float* lds_l = lds_m + WAVES * 32;                         // [waves][2][16]
+    float* lds_ss = lds_l + WAVES * 32;                        // [waves][16]
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
@@ -124,7 +127,7 @@ diff_attention_mfma_kernel(const DiffArgs a) {
 
     const int last_block = a.max_blocks - 1;
     const float scale2 = a.scale * 1.4426950408889634f;            // scores in units of log 2
-    for (int idx = wave; idx < tiles; idx += DMF_WAVES) {
+    for (int idx = wave; idx < tiles; idx += WAVES) {
         const int tile = idx < sink_tiles ? idx : w0 + (idx - sink_tiles);
         const int j0 = tile << 4;
         // keys: lane reads row j0 + r of both maps (a row of the request's pages also where the key is masked)
@@ -251,36 +254,36 @@ diff_attention_mfma_kernel(const DiffArgs a) {
             *reinterpret_cast<dmf_f32x4*>(lds_acc + (((wave * 2 + map) * DVT + c) * 64 + lane) * 4) = acc[map][c];
     }
     __syncthreads();
-    float factor[2][DMF_WAVES], l_all[2];
+    float factor[2][WAVES], l_all[2];
     bool any = true;
 #pragma unroll
     for (int map = 0; map < 2; ++map) {
         float m_all = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < DMF_WAVES; ++w) m_all = fmaxf(m_all, lds_m[(w * 2 + map) * 16 + r]);
+        for (int w = 0; w < WAVES; ++w) m_all = fmaxf(m_all, lds_m[(w * 2 + map) * 16 + r]);
         any = any && m_all > -INFINITY;
         l_all[map] = 0.f;
 #pragma unroll
-        for (int w = 0; w < DMF_WAVES; ++w) {
+        for (int w = 0; w < WAVES; ++w) {
             const float mw = lds_m[(w * 2 + map) * 16 + r];
             factor[map][w] = (m_all > -INFINITY && mw > -INFINITY) ? exp2f(mw - m_all) : 0.f;
             l_all[map] += lds_l[(w * 2 + map) * 16 + r] * factor[map][w];
         }
     }
     // wavefront w joins the maps on the channel tiles w, w + 4, ...
-    constexpr int MINE = (DVT + DMF_WAVES - 1) / DMF_WAVES;
+    constexpr int MINE = (DVT + WAVES - 1) / WAVES;
     dmf_f32x4 o[MINE];
     float ss = 0.f;
 #pragma unroll
     for (int k = 0; k < MINE; ++k) {
-        const int c = wave + k * DMF_WAVES;
+        const int c = wave + k * WAVES;
         o[k] = dmf_f32x4{0.f, 0.f, 0.f, 0.f};
         if (c < DVT && any) {
             dmf_f32x4 sum[2] = {dmf_f32x4{0.f, 0.f, 0.f, 0.f}, dmf_f32x4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
             for (int map = 0; map < 2; ++map)
 #pragma unroll
-                for (int w = 0; w < DMF_WAVES; ++w)
+                for (int w = 0; w < WAVES; ++w)
                     sum[map] += *reinterpret_cast<const dmf_f32x4*>(lds_acc + (((w * 2 + map) * DVT + c) * 64 + lane) * 4) *
                                 factor[map][w];
 #pragma unroll
@@ -296,13 +299,13 @@ diff_attention_mfma_kernel(const DiffArgs a) {
     __syncthreads();
     float total = 0.f;
 #pragma unroll
-    for (int w = 0; w < DMF_WAVES; ++w) total += lds_ss[w * 16 + r];
+    for (int w = 0; w < WAVES; ++w) total += lds_ss[w * 16 + r];
     const float inv = a.out_scale / sqrtf(total / (float)DV + a.eps);
     if (live) {
         bf16* row = a.out + ((int64_t)(t0 + slot_token) * a.nq + head) * DV;
 #pragma unroll
         for (int k = 0; k < MINE; ++k) {
-            const int c = wave + k * DMF_WAVES;
+            const int c = wave + k * WAVES;
             if (c < DVT) {
                 dmf_bf16x4 v = {(bf16)(o[k][0] * inv), (bf16)(o[k][1] * inv), (bf16)(o[k][2] * inv), (bf16)(o[k][3] * inv)};
                 *reinterpret_cast<dmf_bf16x4*>(row + c * 16 + 4 * g) = v;
@@ -311,15 +314,22 @@ diff_attention_mfma_kernel(const DiffArgs a) {
     }
 }
 
-template <int DKT, int DVT>
-static int diff_mfma_launch(const DiffArgs& args, dim3 grid, hipStream_t stream) {
-    const size_t smem = ((size_t)DMF_WAVES * 2 * DVT * 256 + DMF_WAVES * 32 * 2 + DMF_WAVES * 16) * sizeof(float);
+template <int DKT, int DVT, int WAVES>
+static int diff_mfma_launch_waves(const DiffArgs& args, dim3 grid, hipStream_t stream) {
+    const size_t smem = ((size_t)WAVES * 2 * DVT * 256 + WAVES * 32 * 2 + WAVES * 16) * sizeof(float);
+    static_assert(((size_t)WAVES * 2 * DVT * 256 + WAVES * 32 * 2 + WAVES * 16) * sizeof(float) <= 160 * 1024, "LDS of a compute unit");
     if (smem > 64 * 1024)
-        (void)hipFuncSetAttribute((const void*)diff_attention_mfma_kernel<DKT, DVT>,
+        (void)hipFuncSetAttribute((const void*)diff_attention_mfma_kernel<DKT, DVT, WAVES>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipLaunchKernelGGL((diff_attention_mfma_kernel<DKT, DVT>), grid, dim3(DMF_WAVES * 64), smem, stream, args);
+    hipLaunchKernelGGL((diff_attention_mfma_kernel<DKT, DVT, WAVES>), grid, dim3(WAVES * 64), smem, stream, args);
     SOMI_LAUNCH_CHECK("diff_attention_mfma");
     return 0;
+}
+
+template <int DKT, int DVT>
+static int diff_mfma_launch(const DiffArgs& args, dim3 grid, hipStream_t stream) {
+    if (args.listed) return diff_mfma_launch_waves<DKT, DVT, DMF_LISTED_WAVES>(args, grid, stream);
+    return diff_mfma_launch_waves<DKT, DVT, DMF_WAVES>(args, grid, stream);
 }
 
 template <int DKT>
