@@ -99,3 +99,25 @@ def test_the_machines_own_peaks_are_measured_with_the_probes():
     dense = ops.probe_mfma(50, "cuda:0")
     assert dense == ops.probe_mfma(50, "cuda:0", dense=False) > 0
     torch.cuda.synchronize()
+
+
+def test_kamedra_option_runs_both_models_and_leaves_the_default_alone():
+    """``--kamedra`` runs a Kamedra model beside the closest model of equal sizes and prints one JSON line; the sizes'
+    config dictionaries build through the registry like any config.json."""
+    sys.path.insert(0, ROOT)
+    import bench
+    from somi_inference_amd.config import config_from_dict
+    for sizes in bench.KAMEDRA_SIZES:
+        arch, config = config_from_dict(bench.kamedra_config_dict(sizes))
+        assert arch.name == "Kamedra" and len(config.layers) == 6 and config.layers[5].mixer.kv_from == 2
+        arch, config = config_from_dict(bench.closest_config_dict(sizes))
+        assert arch.name == "Qwen2ForCausalLM" and config.num_hidden_layers == 6
+    done = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--kamedra", "1b", "--steps", "16", "--warmup", "2",
+                           "--prefill-tokens", "512", "--context", "1024"], capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-3000:]
+    line = json.loads(done.stdout.strip().splitlines()[-1])
+    for model in ("kamedra", "closest"):
+        assert line[model]["prefill"]["512"]["value"] > 0 and line[model]["decode_b8"]["tok_s"] > 0
+        assert "attention" in line[model]["stages"]["prefill_512"]
+    assert "recurrence" in line["kamedra"]["stages"]["prefill_512"] and line["value"] == line["kamedra"]["decode_b8"]["tok_s"]
+    assert line["prefill_kernels"]["kamedra_attention"]["ms"] > 0 and line["decode_kernels"]["kamedra_recurrence"]["ms"] > 0
