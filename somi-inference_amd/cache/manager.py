@@ -27,7 +27,7 @@ from typing import Hashable
 import numpy as np
 import torch
 
-from ..parts.base import FixedStateSpec, LayerCache, PagedSpec
+from ..parts.base import CompositeSpec, FixedStateSpec, LayerCache, PagedSpec, paged_specs
 from .pool import CacheError, OutOfPages, PagePool
 
 RELEASED = -1     # host-side mark of a logical page a window has passed
@@ -62,7 +62,7 @@ class RequestCache:
 
 
 class CacheManager:
-    def __init__(self, needs: list[PagedSpec | FixedStateSpec | int | None], *, block_size: int,
+    def __init__(self, needs: list[PagedSpec | FixedStateSpec | CompositeSpec | int | None], *, block_size: int,
                  num_blocks: int, max_requests: int, dtype: torch.dtype, device: torch.device | str,
                  allocate_tensors: bool = True) -> None:
         """``block_size``: tokens per page where a spec names no page size of its own.  ``num_blocks``: pages of
@@ -73,42 +73,55 @@ class CacheManager:
         self.dtype, self.device = dtype, torch.device(device)
         self.groups: list[PagedGroup] = []
         self.layer_caches: list[LayerCache | None] = [None] * len(needs)
-        by_need: dict[tuple[int | None, int, int], int] = {}
+        self._by_need: dict[tuple[int | None, int, int], int] = {}
+        self._allocate = bool(allocate_tensors)
         for run, need in enumerate(needs):
-            if isinstance(need, PagedSpec):
-                page_size = int(need.page_size or self.block_size)
-                keep_first = int(need.keep_first) if need.window is not None else 0
-                key = (need.window, page_size, keep_first)
-                if key not in by_need:
-                    pages = self.pool_tokens // page_size
-                    if pages < 1:
-                        raise ValueError(f"a pool of {self.pool_tokens} tokens holds no page of {page_size}")
-                    by_need[key] = len(self.groups)
-                    self.groups.append(PagedGroup(need.window, PagePool(pages), page_size, keep_first))
-                group = by_need[key]
-                self.groups[group].runs.append(run)
-                tensors = {}
-                if allocate_tensors:
-                    pages = self.groups[group].pool.num_pages
-                    tensors = {t.name: torch.zeros((pages, *t.page_shape(page_size)), dtype=t.dtype or dtype,
-                                                   device=self.device) for t in need.tensors}
-                self.layer_caches[run] = LayerCache(need, group, tensors=tensors, page_size=page_size)
-            elif isinstance(need, FixedStateSpec):
-                state = None
-                if allocate_tensors:
-                    # one row more than there are requests: the slot that padding entries of a step use
-                    state = torch.zeros((self.max_requests + 1, *need.shape), dtype=need.dtype, device=self.device)
-                self.layer_caches[run] = LayerCache(need, -1, state=state)
+            if isinstance(need, (PagedSpec, FixedStateSpec, CompositeSpec)):
+                self.layer_caches[run] = self._build(need, run)
         for run, need in enumerate(needs):          # runs that read an earlier run's cache
             if isinstance(need, int) and not isinstance(need, bool):
                 source = self.layer_caches[need]
                 if source is None:
                     raise CacheError(f"run {run} reads the cache of run {need}, which has none")
                 self.layer_caches[run] = LayerCache(source.spec, source.group, tensors=source.tensors,
-                                                    state=source.state, writes=False, page_size=source.page_size)
+                                                    state=source.state, writes=False, page_size=source.page_size,
+                                                    children=source.children)
         self._requests: dict[Hashable, RequestCache] = {}
         self._free_slots = list(range(self.max_requests - 1, -1, -1))
         self.padding_state_slot = self.max_requests       # never handed to a request
+
+    def _build(self, need: "PagedSpec | FixedStateSpec | CompositeSpec", run: int) -> LayerCache:
+        """The cache of one run (or of one part of a run whose mixer is made of several)."""
+        if isinstance(need, CompositeSpec):
+            return LayerCache(need, -1, children={name: self._build(part, run) for name, part in need.parts})
+        if isinstance(need, PagedSpec):
+            page_size = int(need.page_size or self.block_size)
+            keep_first = int(need.keep_first) if need.window is not None else 0
+            key = (need.window, page_size, keep_first)
+            if key not in self._by_need:
+                pages = self.pool_tokens // page_size
+                if pages < 1:
+                    raise ValueError(f"a pool of {self.pool_tokens} tokens holds no page of {page_size}")
+                self._by_need[key] = len(self.groups)
+                self.groups.append(PagedGroup(need.window, PagePool(pages), page_size, keep_first))
+            group = self._by_need[key]
+            self.groups[group].runs.append(run)
+            tensors = {}
+            if self._allocate:
+                pages = self.groups[group].pool.num_pages
+                tensors = {t.name: torch.zeros((pages, *t.page_shape(page_size)), dtype=t.dtype or self.dtype,
+                                               device=self.device) for t in need.tensors}
+            return LayerCache(need, group, tensors=tensors, page_size=page_size)
+        state = None
+        if self._allocate:
+            # one row more than there are requests: the slot that padding entries of a step use
+            state = torch.zeros((self.max_requests + 1, *need.shape), dtype=need.dtype, device=self.device)
+        return LayerCache(need, -1, state=state)
+
+    def state_caches(self) -> list[LayerCache]:
+        """Every cache that holds per-request state of fixed size and is written by its run."""
+        return [leaf for cache in self.layer_caches if cache is not None and cache.writes
+                for leaf in cache.leaves() if leaf.state is not None]
 
     @property
     def pool_tokens(self) -> int:
@@ -122,7 +135,7 @@ class CacheManager:
         def item(kind: torch.dtype | None) -> int:
             return torch.empty((), dtype=kind or dtype).element_size()
         return sum(t.elements_per_token() * int(block_size) * item(t.dtype)
-                   for need in needs if isinstance(need, PagedSpec) for t in need.tensors)
+                   for need in needs for spec in paged_specs(need) for t in spec.tensors)
 
     # --------------------------------------------------------------- requests
     def has(self, request_id: Hashable) -> bool:
@@ -139,9 +152,8 @@ class CacheManager:
         slot = self._free_slots.pop()
         self._requests[request_id] = RequestCache(0, [[] for _ in self.groups], slot,
                                                   [np.zeros(16, dtype=np.int32) for _ in self.groups])
-        for cache in self.layer_caches:
-            if cache is not None and cache.state is not None and cache.writes:
-                cache.state[slot].zero_()
+        for cache in self.state_caches():
+            cache.state[slot].zero_()
 
     def free(self, request_id: Hashable) -> None:
         """Give back every page and the state slot of a request."""

@@ -5,13 +5,15 @@ from .engine import (DEFAULT_BLOCK_SIZE, DEFAULT_MAX_CONCURRENT, DEFAULT_NUM_BLO
                      EngineConfig, normalize_dtype)
 from .kamedra import KamedraAttention, KamedraConfig, KamedraGLA, KamedraLayer, RotaryScaling
 from .qwen2 import Qwen2Config
+from .rusolorn import RusolornAttention, RusolornConfig, RusolornDeltaRule, RusolornExperts, RusolornLayer
 from .registry import (Architecture, config_from_dict, register_architecture,
                        registered_architectures, resolve_architecture, unregister_architecture)
 
 __all__ = [
     "Architecture", "ConfigError", "DEFAULT_BLOCK_SIZE", "DEFAULT_MAX_CONCURRENT",
     "DEFAULT_NUM_BLOCKS", "EngineConfig", "KamedraAttention", "KamedraConfig", "KamedraGLA", "KamedraLayer", "KeyReader",
-    "ModelConfig", "Qwen2Config", "RotaryScaling",
+    "ModelConfig", "Qwen2Config", "RotaryScaling", "RusolornAttention", "RusolornConfig", "RusolornDeltaRule",
+    "RusolornExperts", "RusolornLayer",
     "architecture_of", "config_from_dict", "normalize_dtype", "read_config_json",
     "register_architecture", "registered_architectures", "resolve_architecture",
     "unregister_architecture",

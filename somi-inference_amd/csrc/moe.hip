@@ -1,0 +1,315 @@
+// Mixture of experts: the router, the grouping of (token, expert) pairs by expert, the experts' products over the
+// grouped rows and the weighted sum.
+//
+//   route      z = W_r h (float32), s = softmax(z); experts come in `groups` equal runs of neighbours, a run scores as
+//              its best expert and only the `keep` best runs stay; of their experts the `top` with the largest s are
+//              chosen, weighted by s over the chosen scores' sum (+ 1e-20).  Ties go to the lower index.
+//   align      the N * top pairs sorted by expert: order[], the experts' offsets and a list of row tiles
+//              (expert, first sorted row, rows) that the products' grids walk.
+//   gate_up    act[p, :] = glu(W_gate[e] h_t, W_up[e] h_t) for the sorted pair p = (t, e)
+//   down       y[pair, :] = w_pair * (W_down[e] act[p, :]), float32, at the pair's own place t * top + j
+//   combine    out[t, :] = sum_j y[t * top + j, :] (+ shared[t, :]), float32, in the order of j
+//
+// glu(g, u) = g' sigmoid(alpha g') (u' + shift) with g' = min(g, limit) and u' = clamp(u, -limit, limit).
+// A row's sums run over K in one fixed order whatever else is in the batch.
+#include "common.h"
+
+#define MOE_MAX_EXPERTS 256
+#define MOE_MAX_TOP 32
+#define MOE_TILE_ROWS 16
+
+__device__ __forceinline__ float clamped_glu(float g, float u, float limit, float alpha, float shift) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-alpha * g)) * (u + shift);
+}
+
+// One workgroup per token.
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const T* __restrict__ x, int64_t row_stride, const float* __restrict__ router, int width, int experts,
+                 int top, int groups, int keep, int* __restrict__ chosen, float* __restrict__ weight) {
+    __shared__ float score[MOE_MAX_EXPERTS];
+    __shared__ int allowed[MOE_MAX_EXPERTS];
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const T* row = x + t * row_stride;
+    for (int e = wave; e < experts; e += 4) {
+        const float* w = router + (int64_t)e * width;
+        float acc = 0.f;
+        for (int i = lane; i < width; i += 64) acc += to_float(row[i]) * w[i];
+        acc = wave_sum(acc);
+        if (lane == 0) score[e] = acc;
+    }
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    float top_z = score[0];
+    for (int e = 1; e < experts; ++e) top_z = fmaxf(top_z, score[e]);
+    float total = 0.f;
+    for (int e = 0; e < experts; ++e) {
+        score[e] = expf(score[e] - top_z);
+        total += score[e];
+    }
+    for (int e = 0; e < experts; ++e) {
+        score[e] /= total;
+        allowed[e] = 0;
+    }
+    const int per = experts / groups;
+    // the keep best runs, one at a time (a run already taken is marked through its first expert's flag)
+    for (int round = 0; round < keep; ++round) {
+        int best = -1;
+        float best_score = -1.f;
+        for (int g = 0; g < groups; ++g) {
+            if (allowed[g * per]) continue;
+            float s = score[g * per];
+            for (int j = 1; j < per; ++j) s = fmaxf(s, score[g * per + j]);
+            if (s > best_score) {
+                best_score = s;
+                best = g;
+            }
+        }
+        if (best < 0) break;
+        for (int j = 0; j < per; ++j) allowed[best * per + j] = 1;
+    }
+    int picks[MOE_MAX_TOP];
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) {
+        int best = -1;
+        float best_score = -1.f;
+        for (int e = 0; e < experts; ++e)
+            if (allowed[e] == 1 && score[e] > best_score) {
+                best_score = score[e];
+                best = e;
+            }
+        if (best < 0) {          // scores that compare with nothing (not a number): any expert, weight as it comes
+            best = 0;
+            best_score = score[0];
+        }
+        picks[j] = best;
+        allowed[best] = 2;
+        sum += best_score;
+    }
+    for (int j = 0; j < top; ++j) {
+        chosen[t * top + j] = picks[j];
+        weight[t * top + j] = score[picks[j]] / (sum + 1e-20f);
+    }
+}
+
+extern "C" int somi_moe_route(const void* x, int dtype, int64_t row_stride, const float* router, int n_tokens, int width,
+                              int experts, int top, int groups, int keep, int* chosen, float* weight,
+                              hipStream_t stream) {
+    SOMI_REQUIRE(n_tokens >= 0 && width > 0 && experts > 0 && experts <= MOE_MAX_EXPERTS, "moe_route: %d experts, 1 to %d are supported",
+                 experts, MOE_MAX_EXPERTS);
+    SOMI_REQUIRE(groups >= 1 && experts % groups == 0 && keep >= 1 && keep <= groups, "moe_route: %d groups (keep %d) do not divide %d experts",
+                 groups, keep, experts);
+    SOMI_REQUIRE(top >= 1 && top <= MOE_MAX_TOP && top <= keep * (experts / groups), "moe_route: top %d does not fit the kept experts", top);
+    if (n_tokens == 0) return 0;
+    if (dtype == SOMI_F32)
+        hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, (const float*)x, row_stride, router,
+                           width, experts, top, groups, keep, chosen, weight);
+    else if (dtype == SOMI_BF16)
+        hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(n_tokens), dim3(256), 0, stream, (const bf16*)x, row_stride, router,
+                           width, experts, top, groups, keep, chosen, weight);
+    else
+        return somi_fail("moe_route: unknown dtype %d", dtype);
+    SOMI_LAUNCH_CHECK("moe_route");
+    return 0;
+}
+
+// One workgroup.  tiles: [max_tiles, 3] = (expert or -1, first sorted row, rows).
+__global__ void __launch_bounds__(1024)
+moe_align_kernel(const int* __restrict__ chosen, int pairs, int experts, int tile_rows, int max_tiles,
+                 int* __restrict__ order, int* __restrict__ offsets, int* __restrict__ tiles) {
+    __shared__ int count[MOE_MAX_EXPERTS];
+    __shared__ int cursor[MOE_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < experts; e += 1024) count[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += 1024) atomicAdd(&count[chosen[p]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0, tile = 0;
+        for (int e = 0; e < experts; ++e) {
+            offsets[e] = at;
+            cursor[e] = at;
+            for (int r = 0; r < count[e] && tile < max_tiles; r += tile_rows, ++tile) {
+                tiles[tile * 3] = e;
+                tiles[tile * 3 + 1] = at + r;
+                tiles[tile * 3 + 2] = count[e] - r < tile_rows ? count[e] - r : tile_rows;
+            }
+            at += count[e];
+        }
+        offsets[experts] = at;
+        for (; tile < max_tiles; ++tile) {
+            tiles[tile * 3] = -1;
+            tiles[tile * 3 + 1] = 0;
+            tiles[tile * 3 + 2] = 0;
+        }
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += 1024) order[atomicAdd(&cursor[chosen[p]], 1)] = p;
+}
+
+extern "C" int somi_moe_max_tiles(int pairs, int experts, int tile_rows) {
+    return ceil_div(pairs, tile_rows) + experts;
+}
+
+extern "C" int somi_moe_align(const int* chosen, int pairs, int experts, int tile_rows, int max_tiles, int* order,
+                              int* offsets, int* tiles, hipStream_t stream) {
+    SOMI_REQUIRE(pairs >= 0 && experts > 0 && experts <= MOE_MAX_EXPERTS && tile_rows > 0, "moe_align: bad sizes");
+    SOMI_REQUIRE(max_tiles >= somi_moe_max_tiles(pairs, experts, tile_rows), "moe_align: %d tiles cannot hold %d pairs of %d experts",
+                 max_tiles, pairs, experts);
+    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), 0, stream, chosen, pairs, experts, tile_rows, max_tiles, order,
+                       offsets, tiles);
+    SOMI_LAUNCH_CHECK("moe_align");
+    return 0;
+}
+
+// The experts' products over the sorted rows, plain multiply-adds with float32 sums: a workgroup owns one row tile
+// (MOE_TILE_ROWS sorted rows of one expert) and 64 output columns, K goes through LDS 32 at a time.
+//   GATED: rows are gathered from x by token (pair / top); W: [experts, 2 F, K] (gate rows, then up rows); the end
+//          applies the gated unit and writes act[sorted row, F] in T.
+//   else : rows are act's sorted rows; W: [experts, N, K]; the end multiplies by the pair's weight and writes
+//          y[pair, N] in float32.
+template <typename T, bool GATED>
+__global__ void __launch_bounds__(256)
+moe_product_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w, const int* __restrict__ tiles,
+                   const int* __restrict__ order, const float* __restrict__ pair_weight, int top, int n_out, int K,
+                   float limit, float alpha, float shift, void* __restrict__ out_) {
+    __shared__ float As[MOE_TILE_ROWS][33];
+    __shared__ float Ws[64][33];
+    __shared__ float Us[GATED ? 64 : 1][33];
+    __shared__ int pair_of[MOE_TILE_ROWS];
+    const int expert = tiles[blockIdx.x * 3];
+    if (expert < 0) return;
+    const int first = tiles[blockIdx.x * 3 + 1], rows = tiles[blockIdx.x * 3 + 2];
+    const int col0 = blockIdx.y * 64;
+    const int tid = threadIdx.x;
+    if (tid < MOE_TILE_ROWS) pair_of[tid] = tid < rows ? order[first + tid] : -1;
+    __syncthreads();
+    const int r = tid >> 4, cg = tid & 15;                    // the thread's row and its four columns cg * 4 ..
+    const T* wg = w + (int64_t)expert * (GATED ? 2 : 1) * n_out * K;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f}, acu[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        for (int i = tid; i < MOE_TILE_ROWS * 32; i += 256) {
+            const int rr = i >> 5, kk = i & 31;
+            float v = 0.f;
+            if (rr < rows && k0 + kk < K) {
+                const int64_t src = GATED ? pair_of[rr] / top : first + rr;
+                v = to_float(a[src * a_stride + k0 + kk]);
+            }
+            As[rr][kk] = v;
+        }
+        for (int i = tid; i < 64 * 32; i += 256) {
+            const int cc = i >> 5, kk = i & 31;
+            const bool in = col0 + cc < n_out && k0 + kk < K;
+            Ws[cc][kk] = in ? to_float(wg[(int64_t)(col0 + cc) * K + k0 + kk]) : 0.f;
+            if (GATED) Us[cc][kk] = in ? to_float(wg[(int64_t)(n_out + col0 + cc) * K + k0 + kk]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int kk = 0; kk < 32; ++kk) {
+            const float av = As[r][kk];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[j] += av * Ws[cg * 4 + j][kk];
+                if (GATED) acu[j] += av * Us[cg * 4 + j][kk];
+            }
+        }
+        __syncthreads();
+    }
+    if (r >= rows) return;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int c = col0 + cg * 4 + j;
+        if (c >= n_out) continue;
+        if (GATED) {
+            ((T*)out_)[(int64_t)(first + r) * n_out + c] = from_float<T>(clamped_glu(acc[j], acu[j], limit, alpha, shift));
+        } else {
+            const int pair = pair_of[r];
+            ((float*)out_)[(int64_t)pair * n_out + c] = pair_weight[pair] * acc[j];
+        }
+    }
+}
+
+extern "C" int somi_moe_product(const void* a, int64_t a_stride, const void* w, int dtype, int gated, const int* tiles,
+                                int max_tiles, const int* order, const float* pair_weight, int top, int n_out, int K,
+                                float limit, float alpha, float shift, void* out, hipStream_t stream) {
+    SOMI_REQUIRE(max_tiles >= 0 && n_out > 0 && K > 0 && top > 0 && a_stride >= K, "moe_product: bad sizes");
+    if (max_tiles == 0) return 0;
+    const dim3 grid(max_tiles, ceil_div(n_out, 64));
+    SOMI_REQUIRE(grid.y <= 65535, "moe_product: too many columns");
+#define SOMI_MOE(T, G)                                                                                                   \
+    hipLaunchKernelGGL((moe_product_kernel<T, G>), grid, dim3(256), 0, stream, (const T*)a, a_stride, (const T*)w, tiles, order, \
+                       pair_weight, top, n_out, K, limit, alpha, shift, out)
+    if (dtype == SOMI_F32) {
+        if (gated) SOMI_MOE(float, true); else SOMI_MOE(float, false);
+    } else if (dtype == SOMI_BF16) {
+        if (gated) SOMI_MOE(bf16, true); else SOMI_MOE(bf16, false);
+    } else {
+        return somi_fail("moe_product: unknown dtype %d", dtype);
+    }
+#undef SOMI_MOE
+    SOMI_LAUNCH_CHECK("moe_product");
+    return 0;
+}
+
+// out[t, :] = sum_j y[t * top + j, :] (+ shared[t, :]).
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_combine_kernel(const float* __restrict__ y, const T* __restrict__ shared_rows, int top, int width,
+                   float* __restrict__ out) {
+    const int64_t t = blockIdx.x;
+    for (int c = threadIdx.x; c < width; c += 256) {
+        float acc = 0.f;
+        for (int j = 0; j < top; ++j) acc += y[(t * top + j) * width + c];
+        if (shared_rows != nullptr) acc += to_float(shared_rows[t * width + c]);
+        out[t * width + c] = acc;
+    }
+}
+
+extern "C" int somi_moe_combine(const float* y, const void* shared_rows, int shared_dtype, int n_tokens, int top, int width,
+                                float* out, hipStream_t stream) {
+    SOMI_REQUIRE(n_tokens >= 0 && top > 0 && width > 0, "moe_combine: bad sizes");
+    if (n_tokens == 0) return 0;
+    if (shared_rows == nullptr || shared_dtype == SOMI_F32)
+        hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, y, (const float*)shared_rows, top,
+                           width, out);
+    else if (shared_dtype == SOMI_BF16)
+        hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3(n_tokens), dim3(256), 0, stream, y, (const bf16*)shared_rows, top,
+                           width, out);
+    else
+        return somi_fail("moe_combine: unknown dtype %d", shared_dtype);
+    SOMI_LAUNCH_CHECK("moe_combine");
+    return 0;
+}
+
+// The gated unit on a dense product's rows [gate (F) | up (F)] -> [F].
+template <typename T>
+__global__ void __launch_bounds__(256)
+clamped_glu_kernel(const T* __restrict__ gate_up, int F, float limit, float alpha, float shift, T* __restrict__ out,
+                   int64_t count) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256) {
+        const int64_t t = i / F;
+        const int c = (int)(i - t * F);
+        out[i] = from_float<T>(clamped_glu(to_float(gate_up[t * 2 * F + c]), to_float(gate_up[t * 2 * F + F + c]), limit,
+                                           alpha, shift));
+    }
+}
+
+extern "C" int somi_clamped_glu(const void* gate_up, int dtype, int n_tokens, int F, float limit, float alpha, float shift,
+                                void* out, hipStream_t stream) {
+    SOMI_REQUIRE(n_tokens >= 0 && F > 0, "clamped_glu: bad sizes");
+    if (n_tokens == 0) return 0;
+    const int64_t count = (int64_t)n_tokens * F;
+    const int grid = (int)(ceil_div64(count, 256) < 65536 ? ceil_div64(count, 256) : 65536);
+    if (dtype == SOMI_F32)
+        hipLaunchKernelGGL(clamped_glu_kernel<float>, dim3(grid), dim3(256), 0, stream, (const float*)gate_up, F, limit, alpha,
+                           shift, (float*)out, count);
+    else if (dtype == SOMI_BF16)
+        hipLaunchKernelGGL(clamped_glu_kernel<bf16>, dim3(grid), dim3(256), 0, stream, (const bf16*)gate_up, F, limit, alpha,
+                           shift, (bf16*)out, count);
+    else
+        return somi_fail("clamped_glu: unknown dtype %d", dtype);
+    SOMI_LAUNCH_CHECK("clamped_glu");
+    return 0;
+}

@@ -156,8 +156,7 @@ class ModelRunner:
         # once outside a capture: lazy initialisation (library handles, first allocations) must
         # not happen while the stream is being recorded.  What the step writes into pages is simply
         # written again by the replay; recurrent state that the step advances is put back first.
-        stateful = [cache for cache in self.cache.layer_caches
-                    if cache is not None and cache.state is not None and cache.writes]
+        stateful = self.cache.state_caches()
         slots = static.batch.state_slots.to(torch.int64) if stateful else None
         before = [cache.state.index_select(0, slots) for cache in stateful]
         self.model.forward(static.batch, self.cache.layer_caches)

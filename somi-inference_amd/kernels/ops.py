@@ -919,3 +919,251 @@ def diff_attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
         _ptr(token_list), _ptr(token_entry), _ptr(positions), n_list, nq, nkv, dk, dv, page_size, int(window),
         int(keep_first), ctypes.c_float(scale), ctypes.c_float(lam), ctypes.c_float(eps), ctypes.c_float(out_scale),
         _ptr(out), _stream()))
+
+
+# ------------------------------------------------------------------ the parallel block, its norm and its joins
+def dynamic_tanh(h: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, alpha: torch.Tensor,
+                 out_dtype: torch.dtype) -> torch.Tensor:
+    """tanh(alpha * h) * weight + bias over float32 rows -> rows in ``out_dtype``; ``alpha`` is one float32 number on
+    the device."""
+    _need(h, "residual rows", torch.float32)
+    n, hidden = h.shape
+    _need(weight, "norm weight", torch.float32, (hidden,))
+    _need(bias, "norm bias", torch.float32, (hidden,))
+    _need(alpha, "norm alpha", torch.float32)
+    if alpha.numel() != 1:
+        raise KernelError("dynamic_tanh: alpha is one number")
+    out = torch.empty((n, hidden), dtype=out_dtype, device=h.device)
+    _check(library().somi_dyt(_ptr(h), _ptr(weight), _ptr(bias), _ptr(alpha), _ptr(out), dtype_code(out_dtype), n, hidden,
+                              _stream()))
+    return out
+
+
+def scaled_add(h: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None, mult: float,
+               copy_dtype: torch.dtype | None = None) -> torch.Tensor | None:
+    """h += mult * (a + b) in place on float32 rows (``b`` may be None); with ``copy_dtype`` the new rows are also
+    returned in that dtype."""
+    _need(h, "residual rows", torch.float32)
+    _need(a, "delta", torch.float32, tuple(h.shape))
+    if b is not None:
+        _need(b, "second delta", torch.float32, tuple(h.shape))
+    copy = torch.empty(h.shape, dtype=copy_dtype, device=h.device) if copy_dtype is not None else None
+    _check(library().somi_scaled_add(_ptr(h), _ptr(a), _ptr(b), ctypes.c_float(mult), _ptr(copy),
+                                     dtype_code(copy_dtype) if copy_dtype is not None else 0, ctypes.c_int64(h.numel()),
+                                     _stream()))
+    return copy
+
+
+def normed_pair_mean(left: torch.Tensor, right: torch.Tensor, left_weight: torch.Tensor, right_weight: torch.Tensor,
+                     eps: float) -> torch.Tensor:
+    """(left / rms(left) * left_weight + right / rms(right) * right_weight) / 2 per row -> float32."""
+    _need(left, "left rows")
+    n, width = left.shape
+    _need(right, "right rows", left.dtype, (n, width))
+    _need(left_weight, "left weight", torch.float32, (width,))
+    _need(right_weight, "right weight", torch.float32, (width,))
+    out = torch.empty((n, width), dtype=torch.float32, device=left.device)
+    _check(library().somi_normed_pair_mean(_ptr(left), _ptr(right), dtype_code(left.dtype), _ptr(left_weight),
+                                           _ptr(right_weight), ctypes.c_float(eps), _ptr(out), n, width, _stream()))
+    return out
+
+
+def normed_add(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, mult: float,
+               copy_dtype: torch.dtype | None = None) -> torch.Tensor | None:
+    """h += mult * y / rms(y) * weight in place on float32 rows; with ``copy_dtype`` the new rows are also returned."""
+    _need(h, "residual rows", torch.float32)
+    n, width = h.shape
+    _need(y, "rows to add", torch.float32, (n, width))
+    _need(weight, "norm weight", torch.float32, (width,))
+    copy = torch.empty(h.shape, dtype=copy_dtype, device=h.device) if copy_dtype is not None else None
+    _check(library().somi_normed_add(_ptr(h), _ptr(y), _ptr(weight), ctypes.c_float(eps), ctypes.c_float(mult), _ptr(copy),
+                                     dtype_code(copy_dtype) if copy_dtype is not None else 0, n, width, _stream()))
+    return copy
+
+
+def gated_table_rows(gate: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, offset: int) -> torch.Tensor:
+    """gelu_tanh(gate[t, c]) * table[ids[t], offset + c] -> [N, dim] in the gate's dtype."""
+    _need(gate, "gate rows")
+    n, dim = gate.shape
+    _need(table, "table", gate.dtype)
+    _need(ids, "token ids", torch.int32, (n,))
+    if table.dim() != 2 or offset < 0 or offset + dim > table.shape[1]:
+        raise KernelError(f"gated_table_rows: columns {offset}..{offset + dim} do not fit a table of {tuple(table.shape)}")
+    out = torch.empty_like(gate)
+    _check(library().somi_gated_table_rows(_ptr(gate), _ptr(table), dtype_code(gate.dtype), _ptr(ids), table.shape[0],
+                                           table.shape[1], int(offset), dim, _ptr(out), n, _stream()))
+    return out
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """x *= factor in place on float32 values."""
+    _need(x, "values", torch.float32)
+    _check(library().somi_scale_f32(_ptr(x), ctypes.c_float(factor), ctypes.c_int64(x.numel()), _stream()))
+    return x
+
+
+def qk_norm_store(rows: torch.Tensor, slots: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, eps: float,
+                  nq: int, nkv: int, head_dim: int, tied: bool, k_cache: torch.Tensor, v_cache: torch.Tensor) -> None:
+    """RMS norm of a token's whole q projection (in place) and whole k projection (into the key pages), each with a
+    weight of the projection's size; the value pages get the row's value heads or, ``tied``, the keys as projected.
+    rows: [N, (nq + nkv (+ nkv)) * D]."""
+    _need(rows, "q/k rows")
+    n = rows.shape[0]
+    if rows.shape[1] != (nq + (1 if tied else 2) * nkv) * head_dim:
+        raise KernelError(f"qk_norm_store: rows of {rows.shape[1]} do not hold {nq} + {nkv} heads of {head_dim}")
+    _need(slots, "slot mapping", torch.int32, (n,))
+    _need(q_weight, "q norm weight", torch.float32, (nq * head_dim,))
+    _need(k_weight, "k norm weight", torch.float32, (nkv * head_dim,))
+    _need(k_cache, "k cache", rows.dtype)
+    if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != head_dim:
+        raise KernelError(f"qk_norm_store: cache shape {tuple(k_cache.shape)} != [pages, {nkv}, page, {head_dim}]")
+    _need(v_cache, "v cache", rows.dtype, _v_shape(k_cache))
+    _check(library().somi_qk_norm_store(_ptr(rows), dtype_code(rows.dtype), ctypes.c_int64(rows.shape[1]), _ptr(slots),
+                                        _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps), n, nq, nkv, head_dim,
+                                        1 if tied else 0, _ptr(k_cache), _ptr(v_cache), k_cache.shape[2], _stream()))
+
+
+# ------------------------------------------------------------------------------------------ the gated delta rule
+DELTA_MAX_TAPS = 9
+
+
+def delta_prepare(rows: torch.Tensor, ab: torch.Tensor, taps: torch.Tensor, conv_state: torch.Tensor, step,
+                  a_log: torch.Tensor, dt_bias: torch.Tensor, groups: int, heads: int, dim: int, vdim: int
+                  ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """What the recurrence reads, in float32: (qkv [N, 2 G dim + H vdim], beta [N, H], decay [N, H]).  rows: the tokens'
+    projections [q | k | v | ...]; ab: [N, 2 H] float32 (beta's, then the decay's projection); taps: [C, taps] float32;
+    conv_state: [slots, taps - 1, C] float32, read and then advanced by the step's entries."""
+    _need(rows, "projected rows")
+    n = rows.shape[0]
+    channels = 2 * groups * dim + heads * vdim
+    if rows.shape[1] < channels:
+        raise KernelError(f"delta_prepare: rows of {rows.shape[1]} hold fewer than {channels} channels")
+    _need(ab, "beta/decay projections", torch.float32, (n, 2 * heads))
+    _need(taps, "convolution taps", torch.float32)
+    if taps.dim() != 2 or taps.shape[0] != channels or not 1 <= taps.shape[1] <= DELTA_MAX_TAPS:
+        raise KernelError(f"delta_prepare: taps {tuple(taps.shape)} != [{channels}, 1..{DELTA_MAX_TAPS}]")
+    width = taps.shape[1]
+    _need(conv_state, "convolution state", torch.float32)
+    if tuple(conv_state.shape[1:]) != (max(width - 1, 1), channels):
+        raise KernelError(f"delta_prepare: convolution state {tuple(conv_state.shape)} != [slots, {max(width - 1, 1)}, {channels}]")
+    entries = step.state_slots.numel()
+    _need(step.token_entry, "token entries", torch.int32, (n,))
+    _need(step.entry_start, "entry offsets", torch.int32, (entries + 1,))
+    _need(a_log, "decay rates", torch.float32, (heads,))
+    _need(dt_bias, "decay biases", torch.float32, (heads,))
+    qkv = torch.empty((n, channels), dtype=torch.float32, device=rows.device)
+    beta = torch.empty((n, heads), dtype=torch.float32, device=rows.device)
+    decay = torch.empty((n, heads), dtype=torch.float32, device=rows.device)
+    _check(library().somi_delta_prepare(
+        _ptr(rows), dtype_code(rows.dtype), ctypes.c_int64(rows.stride(0)), _ptr(ab), _ptr(taps), width, _ptr(conv_state),
+        _ptr(step.token_entry), _ptr(step.entry_start), _ptr(step.state_slots), _ptr(a_log), _ptr(dt_bias), n, entries,
+        groups, heads, dim, vdim, _ptr(qkv), _ptr(beta), _ptr(decay), _stream()))
+    return qkv, beta, decay
+
+
+def delta_scan(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, entry_start: torch.Tensor,
+               state_slots: torch.Tensor, state: torch.Tensor, groups: int) -> torch.Tensor:
+    """The recurrence S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q per head over every entry's tokens, from
+    and into ``state[state_slots[e]]`` ([slots, heads, dim, vdim] float32) -> o [N, heads, vdim] float32."""
+    _need(state, "recurrent state", torch.float32)
+    _, heads, dim, vdim = state.shape
+    n = qkv.shape[0]
+    _need(qkv, "q/k/v", torch.float32, (n, 2 * groups * dim + heads * vdim))
+    _need(beta, "beta", torch.float32, (n, heads))
+    _need(decay, "decay", torch.float32, (n, heads))
+    entries = state_slots.numel()
+    _need(entry_start, "entry offsets", torch.int32, (entries + 1,))
+    _need(state_slots, "state slots", torch.int32, (entries,))
+    o = torch.empty((n, heads, vdim), dtype=torch.float32, device=qkv.device)
+    _check(library().somi_delta_scan(_ptr(qkv), _ptr(beta), _ptr(decay), _ptr(entry_start), _ptr(state_slots), _ptr(state),
+                                     entries, groups, heads, dim, vdim, _ptr(o), _stream()))
+    return o
+
+
+# ------------------------------------------------------------------------------------------ mixture of experts
+MOE_TILE_ROWS = 16
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, top: int, groups: int, keep: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Chosen experts [N, top] int32 and their weights [N, top] float32 (softmax scores in float32, the ``keep`` best of
+    ``groups`` runs of neighbouring experts, the ``top`` best experts of those, weights over their sum)."""
+    _need(x, "rows")
+    n, width = x.shape
+    _need(router, "router", torch.float32)
+    if router.dim() != 2 or router.shape[1] != width:
+        raise KernelError(f"moe_route: router {tuple(router.shape)} does not fit rows of {width}")
+    chosen = torch.empty((n, top), dtype=torch.int32, device=x.device)
+    weight = torch.empty((n, top), dtype=torch.float32, device=x.device)
+    _check(library().somi_moe_route(_ptr(x), dtype_code(x.dtype), ctypes.c_int64(x.stride(0)), _ptr(router), n, width,
+                                    router.shape[0], int(top), int(groups), int(keep), _ptr(chosen), _ptr(weight), _stream()))
+    return chosen, weight
+
+
+def moe_align(chosen: torch.Tensor, experts: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The (token, expert) pairs sorted by expert: (order [pairs] int32, offsets [experts + 1] int32, tiles [T, 3] int32
+    = (expert or -1, first sorted row, rows) for row tiles of MOE_TILE_ROWS)."""
+    _need(chosen, "chosen experts", torch.int32)
+    pairs = chosen.numel()
+    max_tiles = library().somi_moe_max_tiles(pairs, int(experts), MOE_TILE_ROWS)
+    order = torch.empty((pairs,), dtype=torch.int32, device=chosen.device)
+    offsets = torch.empty((experts + 1,), dtype=torch.int32, device=chosen.device)
+    tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=chosen.device)
+    _check(library().somi_moe_align(_ptr(chosen), pairs, int(experts), MOE_TILE_ROWS, max_tiles, _ptr(order), _ptr(offsets),
+                                    _ptr(tiles), _stream()))
+    return order, offsets, tiles
+
+
+def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, top: int,
+                limit: float, alpha: float, shift: float) -> torch.Tensor:
+    """act[p] = glu(W_gate[e] x[t], W_up[e] x[t]) for the sorted pairs p = (t, e); gate_up: [experts, 2 F, K], gate rows
+    first -> [pairs, F]."""
+    _need(x, "rows")
+    _need(gate_up, "gate/up matrices", x.dtype)
+    experts, two_f, k = gate_up.shape
+    if x.shape[1] != k or two_f % 2:
+        raise KernelError(f"moe_gate_up: matrices {tuple(gate_up.shape)} do not fit rows of {x.shape[1]}")
+    pairs = order.numel()
+    act = torch.empty((pairs, two_f // 2), dtype=x.dtype, device=x.device)
+    _check(library().somi_moe_product(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(gate_up), dtype_code(x.dtype), 1, _ptr(tiles),
+                                      tiles.shape[0], _ptr(order), None, int(top), two_f // 2, k, ctypes.c_float(limit),
+                                      ctypes.c_float(alpha), ctypes.c_float(shift), _ptr(act), _stream()))
+    return act
+
+
+def moe_down(act: torch.Tensor, down: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, weight: torch.Tensor,
+             top: int) -> torch.Tensor:
+    """y[pair] = weight[pair] * W_down[e] act[p] -> [pairs, width] float32, at the pairs' own places."""
+    _need(act, "activations")
+    _need(down, "down matrices", act.dtype)
+    experts, width, k = down.shape
+    if act.shape[1] != k:
+        raise KernelError(f"moe_down: matrices {tuple(down.shape)} do not fit activations of {act.shape[1]}")
+    _need(weight, "pair weights", torch.float32)
+    y = torch.empty((order.numel(), width), dtype=torch.float32, device=act.device)
+    _check(library().somi_moe_product(_ptr(act), ctypes.c_int64(act.stride(0)), _ptr(down), dtype_code(act.dtype), 0, _ptr(tiles),
+                                      tiles.shape[0], _ptr(order), _ptr(weight), int(top), width, k, ctypes.c_float(0.0),
+                                      ctypes.c_float(0.0), ctypes.c_float(0.0), _ptr(y), _stream()))
+    return y
+
+
+def moe_combine(y: torch.Tensor, top: int, shared: torch.Tensor | None) -> torch.Tensor:
+    """out[t] = sum_j y[t * top + j] (+ shared[t]) -> [N, width] float32."""
+    _need(y, "expert outputs", torch.float32)
+    pairs, width = y.shape
+    n = pairs // top
+    if shared is not None:
+        _need(shared, "shared expert rows", None, (n, width))
+    out = torch.empty((n, width), dtype=torch.float32, device=y.device)
+    _check(library().somi_moe_combine(_ptr(y), _ptr(shared), dtype_code(shared.dtype) if shared is not None else 0, n, int(top),
+                                      width, _ptr(out), _stream()))
+    return out
+
+
+def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, shift: float) -> torch.Tensor:
+    """g' sigmoid(alpha g') (u' + shift) with g' = min(g, limit), u' = clamp(u, -limit, limit) on rows [g | u]."""
+    _need(gate_up, "gate/up rows")
+    n, two_f = gate_up.shape
+    out = torch.empty((n, two_f // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _check(library().somi_clamped_glu(_ptr(gate_up), dtype_code(gate_up.dtype), n, two_f // 2, ctypes.c_float(limit),
+                                      ctypes.c_float(alpha), ctypes.c_float(shift), _ptr(out), _stream()))
+    return out

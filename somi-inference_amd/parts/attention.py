@@ -18,8 +18,8 @@ import torch
 from ..kernels import attention as attention_kernels
 from ..kernels import ops
 from ..kernels.stages import stage
-from ..weights.spec import MATRIX, VECTOR, WeightSpec
-from .base import Fetch, LayerCache, Mixer, PagedKVSpec, PartSpec, Runtime
+from ..weights.spec import MATRIX, VECTOR, Init, WeightSpec
+from .base import Fetch, LayerCache, Mixer, PagedKVSpec, PartSpec, PositionEncoding, Runtime
 from .linear import NormedRows, Projection
 from .registry import build_part
 
@@ -32,11 +32,26 @@ class GroupedQueryAttention(Mixer):
     def __init__(self, prefix: str, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: PartSpec, qkv_bias: bool = True, out_bias: bool = False,
                  window: int | None = None, scale: float | None = None, shares_cache: bool = False,
-                 names: dict[str, str] | None = None) -> None:
+                 names: dict[str, str] | None = None, values: str = "projection", qk_norm: str | None = None,
+                 norm_eps: float = 1e-6, suffix: str = "weight") -> None:
         """``names``: what the checkpoint calls this part's tensors, role -> name under the prefix.  Roles: ``q``,
         ``k``, ``v``, ``o`` (defaults ``q_proj`` ... ``o_proj``), ``position`` (``rotary_emb``), and ``qkv`` for a
-        checkpoint that stores the three projections as one matrix, q rows first, then k, then v."""
+        checkpoint that stores the three projections as one matrix, q rows first, then k, then v.
+
+        ``values``: "projection" (a value projection of its own) or "keys" (there is none: a token's values are its
+        keys as projected, before any norm).  ``qk_norm``: None, or "projection": q and k are each RMS-normed over the
+        whole projection, all heads at once, with a weight of that size (roles ``q_norm``, ``k_norm``; ``norm_eps``
+        inside the root).  ``suffix``: what follows a matrix's name in the checkpoint (empty: nothing; a bias is then
+        ``<name>.bias`` all the same)."""
         super().__init__(prefix)
+        if values not in ("projection", "keys") or qk_norm not in (None, "projection"):
+            raise ValueError(f"{prefix}: values must be 'projection' or 'keys' and qk_norm None or 'projection', got "
+                             f"{values!r} and {qk_norm!r}")
+        self.values_are_keys, self.qk_norm, self.norm_eps = values == "keys", qk_norm, float(norm_eps)
+        self.suffix = str(suffix)
+        if (self.values_are_keys or qk_norm) and (shares_cache or qkv_bias or "qkv" in (names or {})):
+            raise ValueError(f"{prefix}: values from the keys and a norm over the projections come without biases, "
+                             f"a merged q/k/v matrix or a borrowed cache")
         unknown = set(names or {}) - set(self.ROLES) - {"qkv"}
         if unknown:
             raise ValueError(f"{prefix}: unknown tensor roles {sorted(unknown)}; known: {sorted(self.ROLES)} and 'qkv'")
@@ -54,7 +69,11 @@ class GroupedQueryAttention(Mixer):
         if getattr(self.position, "pairing", "half") != "half":
             raise ValueError(f"{prefix}: this part's kernels rotate channel j with j + rotary_dim / 2 only")
 
-    ROLES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "position": "rotary_emb"}
+    ROLES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "position": "rotary_emb",
+             "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
+
+    def _weight(self, name: str) -> str:
+        return self.name(f"{name}.{self.suffix}" if self.suffix else name)
 
     # ------------------------------------------------------------------ weights
     def _projections(self) -> list[tuple[str, int]]:
@@ -64,29 +83,37 @@ class GroupedQueryAttention(Mixer):
             return [(self.names["q"], q_width)]
         if "qkv" in self.names:
             return [(self.names["qkv"], q_width + 2 * kv_width)]
+        if self.values_are_keys:
+            return [(self.names["q"], q_width), (self.names["k"], kv_width)]
         return [(self.names["q"], q_width), (self.names["k"], kv_width), (self.names["v"], kv_width)]
 
     def weight_specs(self) -> list[WeightSpec]:
         specs = []
         for proj, width in self._projections():
-            specs.append(WeightSpec(self.name(f"{proj}.weight"), (width, self.hidden_size), MATRIX))
+            specs.append(WeightSpec(self._weight(proj), (width, self.hidden_size), MATRIX))
             if self.qkv_bias:
                 specs.append(WeightSpec(self.name(f"{proj}.bias"), (width,), VECTOR))
         out = self.names["o"]
-        specs.append(WeightSpec(self.name(f"{out}.weight"), (self.hidden_size, self.num_heads * self.head_dim), MATRIX))
+        specs.append(WeightSpec(self._weight(out), (self.hidden_size, self.num_heads * self.head_dim), MATRIX))
         if self.out_bias:
             specs.append(WeightSpec(self.name(f"{out}.bias"), (self.hidden_size,), VECTOR))
+        if self.qk_norm:
+            specs.append(WeightSpec(self.name(self.names["q_norm"]), (self.num_heads * self.head_dim,), VECTOR, Init(1.0, 0.1)))
+            specs.append(WeightSpec(self.name(self.names["k_norm"]), (self.num_kv_heads * self.head_dim,), VECTOR, Init(1.0, 0.1)))
         return specs + self.position.weight_specs()
 
     def load(self, fetch: Fetch, runtime: Runtime) -> None:
         super().load(fetch, runtime)
         names = [p for p, _ in self._projections()]
         self.qkv = Projection.stacked(
-            [fetch(self.name(f"{p}.weight")) for p in names],
+            [fetch(self._weight(p)) for p in names],
             [fetch(self.name(f"{p}.bias")) for p in names] if self.qkv_bias else None, label="q/k/v")
         out = self.names["o"]
-        self.out = Projection(fetch(self.name(f"{out}.weight")),
+        self.out = Projection(fetch(self._weight(out)),
                               fetch(self.name(f"{out}.bias")) if self.out_bias else None, label="o")
+        if self.qk_norm:
+            self.q_norm_weight = fetch(self.name(self.names["q_norm"]))
+            self.k_norm_weight = fetch(self.name(self.names["k_norm"]))
         self.position.load(fetch, runtime)
 
     def flops(self, tokens: int, attended: int) -> float:
@@ -108,6 +135,8 @@ class GroupedQueryAttention(Mixer):
         view = step.paged[cache.group]
         nkv_new = 0 if self.shares_cache else self.num_kv_heads
         rotation = self.position.rotation_table()
+        if self.qk_norm or self.values_are_keys:
+            return self._forward_normed(x, step, view, cache, rotation)
         with stage(self.qkv.label):
             qkv = self._project_rotate_store(x, step, view, cache, rotation)     # a few rows: one kernel
         if qkv is None:
@@ -126,6 +155,24 @@ class GroupedQueryAttention(Mixer):
                 qkv, self.num_heads, cache.k, cache.v, view.block_table, step,
                 window=self.window or 0, scale=self.scale)
         return self.out.deferred(attended)        # the residual stream may add it in the kernel that computes it
+
+    def _forward_normed(self, x, step, view, cache: LayerCache, rotation):
+        """The path of a norm over the whole projections and of values that are the keys: the product, then one kernel
+        that norms q in place and puts the normed keys and the values into their pages, then attention."""
+        if rotation is not None or type(self.position).encode_qk is not PositionEncoding.encode_qk:
+            raise ValueError(f"{self.prefix}: no kernel rotates after a norm over the whole projection")
+        rows = self.qkv(x)                              # [N, (nq + nkv (+ nkv)) * D]
+        with stage("q/k norm, k/v into pages"):
+            if self.qk_norm:
+                q_weight, k_weight, eps = self.q_norm_weight, self.k_norm_weight, self.norm_eps
+            else:
+                raise ValueError(f"{self.prefix}: values from the keys come with the norm over the projections")
+            ops.qk_norm_store(rows, view.slot_mapping, q_weight, k_weight, eps, self.num_heads, self.num_kv_heads,
+                              self.head_dim, self.values_are_keys, cache.k, cache.v)
+        with stage("attention"):
+            attended = attention_kernels.paged_attention(rows, self.num_heads, cache.k, cache.v, view.block_table, step,
+                                                         window=self.window or 0, scale=self.scale)
+        return self.out.deferred(attended)
 
     def _project_rotate_store(self, x, step, view, cache: LayerCache, rotation) -> torch.Tensor | None:
         """q of the step's tokens, rotated, with k and v in their pages, by the q/k/v product itself (up to 64 rows) or

@@ -125,6 +125,29 @@ class FixedStateSpec:
     dtype: torch.dtype = torch.float32
 
 
+@dataclass(frozen=True)
+class CompositeSpec:
+    """What a mixer made of several mixers keeps: (name, what that mixer keeps) for each of them that keeps
+    anything.  The cache manager builds each as it would for a layer of its own (paged ones join the groups of
+    their window and page size, fixed state gets the request's slot) and hands them out as ``LayerCache.children``."""
+
+    parts: tuple[tuple[str, "PagedSpec | FixedStateSpec | CompositeSpec"], ...]
+
+    def __post_init__(self) -> None:
+        names = [name for name, _ in self.parts]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a composite cache needs at least one part and distinct names, got {names}")
+
+
+def paged_specs(need) -> list[PagedSpec]:
+    """Every paged spec inside ``need`` (itself, or the parts of a composite, in order)."""
+    if isinstance(need, PagedSpec):
+        return [need]
+    if isinstance(need, CompositeSpec):
+        return [spec for _, part in need.parts for spec in paged_specs(part)]
+    return []
+
+
 @dataclass
 class LayerCache:
     """What one run of a layer sees of the cache: the tensors of its call site.
@@ -134,12 +157,19 @@ class LayerCache:
     ``writes`` is False for a layer that reads the cache another layer wrote.
     """
 
-    spec: PagedSpec | FixedStateSpec
+    spec: "PagedSpec | FixedStateSpec | CompositeSpec"
     group: int
     tensors: dict[str, torch.Tensor] = field(default_factory=dict)
     state: torch.Tensor | None = None    # [slots, *shape]
     writes: bool = True
     page_size: int = 0
+    children: dict[str, "LayerCache"] = field(default_factory=dict)   # of a composite spec: name -> that part's cache
+
+    def leaves(self) -> list["LayerCache"]:
+        """The caches that hold tensors: this one, or those of a composite's parts."""
+        if not self.children:
+            return [self]
+        return [leaf for child in self.children.values() for leaf in child.leaves()]
 
     @property
     def k(self) -> torch.Tensor | None:      # [pages, kv_heads, page_size, head_dim]

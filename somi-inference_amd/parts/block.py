@@ -2,6 +2,10 @@
 
 from __future__ import annotations
 
+import torch
+
+from ..kernels import ops
+from ..kernels.stages import stage
 from .base import Block, LayerCache, Part, PartSpec
 from .registry import build_part
 from .residual import ResidualStream
@@ -45,3 +49,48 @@ class PreNormBlock(Block):
             return
         x = stream.normed(self.ffn_norm, lazy=getattr(self.feed_forward, "takes_normed_rows", False))
         stream.add(self.feed_forward.forward(x, step))
+
+
+class ParallelBlock(Block):
+    """One norm, and mixer and feed-forward side by side: with x' = norm(h), ``h += mult * (mixer(x') + ff(x'))``;
+    then, if the layer has one, a per-layer token input adds to h from the token itself (``token_input``, a part of
+    the category of that name with ``add_to(h, x, step, mult)``).  The sum is float32; a layer without a feed-forward
+    adds the mixer alone.  ``names``: the sub-prefixes of the norm, the mixer, the feed-forward and the token input."""
+
+    DEFAULT_NAMES = {"norm": "input_layernorm", "mixer": "self_attn", "feed_forward": "mlp", "token_input": "token_input"}
+
+    def __init__(self, prefix: str, mixer: PartSpec, feed_forward: PartSpec | None, norm: PartSpec,
+                 residual_mult: float = 1.0, token_input: PartSpec | None = None,
+                 names: dict[str, str] | None = None) -> None:
+        super().__init__(prefix)
+        sub = dict(self.DEFAULT_NAMES)
+        sub.update(names or {})
+        self.residual_mult = float(residual_mult)
+        self.norm = build_part("norm", norm, prefix=self.name(sub["norm"]))
+        self.mixer = build_part("mixer", mixer, prefix=self.name(sub["mixer"]))
+        self.feed_forward = (build_part("feed_forward", feed_forward, prefix=self.name(sub["feed_forward"]))
+                             if feed_forward is not None else None)
+        self.token_input = (build_part("token_input", token_input, prefix=self.name(sub["token_input"]))
+                            if token_input is not None else None)
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in self.parts())
+
+    def parts(self) -> list[Part]:
+        return [part for part in (self.norm, self.mixer, self.feed_forward, self.token_input) if part is not None]
+
+    def forward(self, stream: ResidualStream, step, cache: LayerCache | None) -> None:
+        x = stream.normed(self.norm)
+        mixed = _float32_rows(self.mixer.forward(x, step, cache))
+        fed = _float32_rows(self.feed_forward.forward(x, step)) if self.feed_forward is not None else None
+        h = stream.settle()
+        with stage("residual add"):
+            copy = ops.scaled_add(h, mixed, fed, self.residual_mult,
+                                  self.runtime.dtype if self.token_input is not None else None)
+        if self.token_input is not None:
+            self.token_input.add_to(h, copy, step, self.residual_mult)
+
+
+def _float32_rows(y):
+    """A sublayer's output as float32 rows (a promised product is computed, 16-bit rows are widened)."""
+    if hasattr(y, "materialize"):
+        y = y.materialize()
+    return y if y.dtype == torch.float32 else y.to(torch.float32)

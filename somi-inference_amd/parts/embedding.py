@@ -19,11 +19,14 @@ from .base import Fetch, Part, Runtime
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, prefix: str, vocab_size: int, hidden_size: int, tensor: str = "weight") -> None:
-        """``tensor``: what the checkpoint calls the table under the part's prefix."""
+    def __init__(self, prefix: str, vocab_size: int, hidden_size: int, tensor: str = "weight",
+                 scale: float | None = None) -> None:
+        """``tensor``: what the checkpoint calls the table under the part's prefix.  ``scale``: a factor on the
+        embedded rows (a head tied to the table multiplies by the table itself, without it)."""
         super().__init__(prefix)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.tensor = str(tensor)
+        self.scale = float(scale) if scale is not None and float(scale) != 1.0 else None
         self.weight: torch.Tensor | None = None
 
     def weight_specs(self) -> list[WeightSpec]:
@@ -35,7 +38,8 @@ class TokenEmbedding(Part):
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         """[N] int32 -> [N, H] float32 (the residual stream starts in float32)."""
-        return ops.embedding(self.weight, token_ids)
+        h = ops.embedding(self.weight, token_ids)
+        return ops.scale_(h, self.scale) if self.scale is not None else h
 
 
 class LMHead(Part):
