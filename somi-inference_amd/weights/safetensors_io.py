@@ -106,6 +106,6 @@ def write_file(path: str, tensors: dict[str, torch.Tensor], metadata: dict[str, 
         handle.write(struct.pack("<Q", len(blob)))
         handle.write(blob)
         for tensor in tensors.values():
-            host = tensor.detach().contiguous().cpu()
+            host = tensor.detach().contiguous().cpu().reshape(-1)      # a tensor of no dimensions is one element
             handle.write(host.view(torch.uint8).numpy().tobytes() if host.numel() else b"")
     os.replace(tmp, path)

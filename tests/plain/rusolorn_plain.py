@@ -122,10 +122,32 @@ def route(h: torch.Tensor, router: torch.Tensor, top: int, groups: int, keep: in
     return chosen, weight
 
 
-def mixture(h: torch.Tensor, weights: dict, prefix: str, mlp: dict) -> torch.Tensor:
+def routing_margins(h: torch.Tensor, router: torch.Tensor, top: int, groups: int, keep: int) -> torch.Tensor:
+    """Per token, how far the router's decisions are from a tie: the smaller of (the last chosen expert's score over
+    the best allowed expert's that was not chosen) and (the last kept run's score over the best dropped run's), minus
+    one.  A token with a small margin may be routed otherwise by rounding alone."""
+    scores = torch.softmax(h @ router.T, dim=-1)
+    tokens, experts = scores.shape
+    per = experts // groups
+    chosen, _ = route(h, router, top, groups, keep)
+    out = torch.full((tokens,), float("inf"))
+    for t in range(tokens):
+        runs = sorted((float(scores[t, g * per:(g + 1) * per].max()) for g in range(groups)), reverse=True)
+        if keep < groups:
+            out[t] = min(float(out[t]), runs[keep - 1] / runs[keep] - 1.0)
+        kept = sorted(range(groups), key=lambda g: (-float(scores[t, g * per:(g + 1) * per].max()), g))[:keep]
+        rest = [float(scores[t, e]) for e in range(experts) if e // per in kept and e not in chosen[t].tolist()]
+        if rest:
+            out[t] = min(float(out[t]), float(scores[t, chosen[t]].min()) / max(rest) - 1.0)
+    return out
+
+
+def mixture(h: torch.Tensor, weights: dict, prefix: str, mlp: dict, margins: list | None = None) -> torch.Tensor:
     router = mlp["router"]
     groups = router.get("groups") or {"count": 1, "keep": 1}
     chosen, weight = route(h, weights[prefix + ".router"], router["top"], groups["count"], groups["keep"])
+    if margins is not None:
+        margins.append(routing_margins(h, weights[prefix + ".router"], router["top"], groups["count"], groups["keep"]))
     out = torch.zeros(h.shape[0], weights[prefix + ".e0.down"].shape[0])
     for t in range(h.shape[0]):
         for e, w in zip(chosen[t].tolist(), weight[t]):
@@ -143,8 +165,9 @@ def token_side(x: torch.Tensor, tokens: torch.Tensor, weights: dict, layer: int,
     return rms(y, eps) * weights[f"l{layer}.side.norm"]
 
 
-def forward(config: dict, weights: dict, tokens: list[int], keep_layers: bool = False):
-    """Logits [T, vocab] of a whole sequence; with ``keep_layers`` also the residual stream after every layer."""
+def forward(config: dict, weights: dict, tokens: list[int], keep_layers: bool = False, margins: list | None = None):
+    """Logits [T, vocab] of a whole sequence; with ``keep_layers`` also the residual stream after every layer;
+    ``margins`` collects every routed layer's :func:`routing_margins`."""
     ids = torch.tensor(tokens, dtype=torch.long)
     eps, m = config["norm"]["eps"], config.get("residual_mult", 1.0)
     x = weights["embed"][ids] * config["embedding"]["scale"]
@@ -155,7 +178,7 @@ def forward(config: dict, weights: dict, tokens: list[int], keep_layers: bool = 
         h = dynamic_tanh(x, weights, prefix + ".norm1")
         delta = parallel_mixer(h, weights, prefix + ".mix", layer["mixer"], eps)
         if layer.get("mlp"):
-            delta = delta + mixture(h, weights, prefix + ".mlp", layer["mlp"])
+            delta = delta + mixture(h, weights, prefix + ".mlp", layer["mlp"], margins)
         x = x + m * delta
         if side:
             x = x + m * token_side(x, ids, weights, index, side["dim"], eps)
