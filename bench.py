@@ -83,6 +83,44 @@ def closest_config_dict(sizes: str) -> dict:
             "tie_word_embeddings": True, "max_position_embeddings": 32768, "hidden_act": "silu", "attention_bias": False}
 
 
+# layer sizes of Rusolorn models that resemble real ones: (width, attention heads, key/value heads, head size, window,
+# recurrent value heads, recurrent q/k heads, their key size, their value size, taps, experts, experts a token, groups,
+# kept groups, an expert's size, the shared expert's size, columns of the token input, vocabulary).  Six parallel layers.
+RUSOLORN_SIZES = {
+    "1b": (2048, 16, 4, 128, 1024, 16, 8, 128, 128, 4, 32, 4, 8, 4, 512, 1024, 128, 32000),
+    "7b": (4096, 32, 8, 128, 2048, 32, 16, 128, 128, 4, 64, 6, 8, 4, 1024, 2048, 256, 32000),
+}
+RUSOLORN_LAYERS = 6
+
+
+def rusolorn_config_dict(sizes: str) -> dict:
+    (width, heads, kv_heads, dim, window, r_heads, r_groups, r_dim, r_vdim, taps, experts, top, groups, keep, ff, shared,
+     side, vocab) = RUSOLORN_SIZES[sizes]
+    layer = {"type": "parallel",
+             "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                "mask": {"size": window}},
+                       "right": {"heads": r_heads, "kv_heads": r_groups, "dim": r_dim, "vdim": r_vdim, "conv": taps}},
+             "mlp": {"kind": "moe", "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}},
+                     "expert": {"ff": ff, "limit": 7.0}, "shared": {"ff": shared, "limit": 7.0}}}
+    return {"architecture": "Rusolorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+            "residual_mult": 0.5, "token_side": {"dim": side}, "layers": [layer] * RUSOLORN_LAYERS}
+
+
+def rusolorn_closest_config_dict(sizes: str) -> dict:
+    """The closest model the engine had before: a Kamedra model of the same width, attention heads, window, recurrent
+    heads and layers, whose layers take turns between the recurrent mixer and attention (a Rusolorn layer has both side
+    by side) and whose dense feed-forward has the size of the experts a token uses plus the shared one."""
+    (width, heads, kv_heads, dim, window, r_heads, _, r_dim, r_vdim, _, _, top, _, _, ff, shared, _, vocab) = RUSOLORN_SIZES[sizes]
+    dense = {"kind": "dense", "ff": top * ff + shared}
+    recurrent = {"type": "gla", "mlp": dense, "mixer": {"heads": r_heads, "dim": r_dim, "vdim": r_vdim, "tau": 16.0, "rank": 64}}
+    attention = {"type": "attention", "mlp": dense,
+                 "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim // 2, "vdim": dim, "diff": 0.6,
+                           "scale": (dim // 2) ** -0.5, "mask": {"size": window, "keep_first": 0},
+                           "rot": {"base": 500000.0, "dims": dim // 2}}}
+    return {"architecture": "Kamedra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+            "layers": [recurrent, attention] * (RUSOLORN_LAYERS // 2)}
+
+
 # keys of a config.json that name sizes, in the order they are reported under "config" (flat, at most 20 keys)
 SIZE_KEYS = ("hidden_size", "intermediate_size", "num_attention_heads", "num_key_value_heads", "head_dim",
              "vocab_size", "tie_word_embeddings")
@@ -119,6 +157,10 @@ def parse_args() -> argparse.Namespace:
                    help="instead of the default workload: prefill and decode of a Kamedra model (differential attention "
                         "with a window, gated linear attention) at these layer sizes, beside the Qwen2.5-style model of "
                         "equal width, heads, feed-forward and layers, each with its stage times")
+    p.add_argument("--rusolorn", default=None, choices=sorted(RUSOLORN_SIZES), metavar="SIZES",
+                   help="instead of the default workload: prefill and decode of a Rusolorn model (windowed attention "
+                        "beside a gated delta rule, routed experts) at these layer sizes, beside the Kamedra model of "
+                        "equal width, heads, active feed-forward size and layers, each with its stage times")
     p.add_argument("--serving", type=int, default=0, metavar="REQUESTS",
                    help="also run this many requests (prompts of 128 to 2,048 tokens, 256 new tokens each) through "
                         "the scheduler with portions of 512, and report it under 'serving'")
@@ -550,6 +592,71 @@ def run_kamedra(args) -> dict:
     return out
 
 
+def run_rusolorn(args) -> dict:
+    """Prefill and decode of a Rusolorn model beside the closest Kamedra model, with the stage times of both and what
+    the attention, recurrence and feed-forward stages reach of the machine."""
+    (width, heads, kv_heads, dim, window, r_heads, r_groups, r_dim, r_vdim, taps, experts, top, groups, keep, ff, shared,
+     side, vocab) = RUSOLORN_SIZES[args.rusolorn]
+    batches, context, tokens = (8, 64), args.context, args.prefill_tokens
+    out: dict = {}
+    for label, config_dict in (("rusolorn", rusolorn_config_dict(args.rusolorn)),
+                               ("closest", rusolorn_closest_config_dict(args.rusolorn))):
+        bench = Workbench(config_dict, dtype=args.dtype, seed=args.seed, block_size=args.block_size,
+                          pool_tokens=Workbench.pool_tokens(batches, context, tokens), max_requests=max(batches))
+        block: dict = {"prefill": {str(n): bench.prefill_run(n) for n in sorted({512, tokens})}}
+        for batch in batches:
+            run = bench.decode_run(batch, max(POINT_MIN_STEPS, args.steps // 2), max(2, args.warmup // 2), context)
+            block[f"decode_b{batch}"] = {"tok_s": round(run["tok_s"], 1), "ms": round(run["ms"], 4),
+                                        "mean_ctx": round(run["mean_ctx"], 1)}
+        block["stages"] = bench.stage_run(tokens, batches[0], context)
+        print_stage_tables(block["stages"])
+        out[label] = block
+        bench.close()
+    bf16_peak = PEAK_FLOPS["bfloat16"]
+    pairs = sum(min(p + 1, window) for p in range(tokens))
+
+    def stage_ms(block, run, *names):
+        return sum(block["stages"][run].get(name, {}).get("ms", 0.0) for name in names)
+
+    def rate(flops, ms):
+        return {"ms": round(ms, 4), "tflops": round(flops / 1e9 / max(ms, 1e-9), 2),
+                "frac_of_peak": round(flops / 1e3 / max(ms, 1e-9) / bf16_peak * 1e6, 5)}
+    run, layers, half = f"prefill_{tokens}", RUSOLORN_LAYERS, RUSOLORN_LAYERS // 2
+    out["prefill_kernels"] = {
+        "tokens": tokens,
+        # scores and weights times values over the visible pairs (the closest model: two maps of half the key size)
+        "rusolorn_attention": rate(layers * 4.0 * heads * dim * pairs, stage_ms(out["rusolorn"], run, "attention")),
+        "closest_attention": rate(half * 4.0 * heads * (dim // 2 + dim) * pairs, stage_ms(out["closest"], run, "attention")),
+        # per token and head: three passes over the state here (two products, one update), two in the closest model
+        "rusolorn_recurrence": rate(layers * 6.0 * r_heads * r_dim * r_vdim * tokens, stage_ms(out["rusolorn"], run, "recurrence")),
+        "closest_recurrence": rate(half * 4.0 * r_heads * r_dim * r_vdim * tokens, stage_ms(out["closest"], run, "recurrence")),
+        # the routed experts' three matrices over the pairs, against the dense feed-forward's products
+        "rusolorn_experts": rate(layers * 6.0 * tokens * top * ff * width,
+                                 stage_ms(out["rusolorn"], run, "experts gate_up", "experts down")),
+        "closest_feed_forward": rate(layers * 6.0 * tokens * (top * ff + shared) * width,
+                                     stage_ms(out["closest"], run, "gate_up", "down")),
+        "rusolorn_router": {"ms": round(stage_ms(out["rusolorn"], run, "router"), 4)},
+    }
+    run = f"decode_b{batches[0]}_eager"
+
+    def stream(bytes_, ms):
+        return {"ms": round(ms, 4), "gbs": round(bytes_ / 1e6 / max(ms, 1e-9), 1)}
+    seen = min(context, window)
+    used = min(experts, batches[0] * top)          # experts a step touches at most
+    out["decode_kernels"] = {
+        "batch": batches[0], "context": context,
+        "rusolorn_attention": stream(layers * batches[0] * seen * kv_heads * 2 * dim * 2.0, stage_ms(out["rusolorn"], run, "attention")),
+        "closest_attention": stream(half * batches[0] * seen * kv_heads * (dim + dim) * 2.0, stage_ms(out["closest"], run, "attention")),
+        "rusolorn_recurrence": stream(layers * batches[0] * r_heads * r_dim * r_vdim * 4.0 * 2, stage_ms(out["rusolorn"], run, "recurrence")),
+        "closest_recurrence": stream(half * batches[0] * r_heads * r_dim * r_vdim * 4.0 * 2, stage_ms(out["closest"], run, "recurrence")),
+        "rusolorn_experts": stream(layers * used * 3.0 * ff * width * 2.0,
+                                   stage_ms(out["rusolorn"], run, "experts gate_up", "experts down")),
+        "closest_feed_forward": stream(layers * 3.0 * (top * ff + shared) * width * 2.0,
+                                       stage_ms(out["closest"], run, "gate_up", "down")),
+    }
+    return out
+
+
 def main() -> int:
     args = parse_args()
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -564,6 +671,16 @@ def main() -> int:
                 "data": "synthetic: seeded random weights, seeded uniform token ids", "sizes": args.kamedra}
         line.update(run_kamedra(args))
         line["value"] = line["kamedra"][f"decode_b8"]["tok_s"]
+        line["seconds_total"] = round(time.perf_counter() - started, 1)
+        print(json.dumps(line))
+        return 0
+
+    if args.rusolorn:
+        line = {"metric": f"Rusolorn at {args.rusolorn} layer sizes beside the closest Kamedra model: prefill and decode",
+                "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                "data": "synthetic: seeded random weights, seeded uniform token ids", "sizes": args.rusolorn}
+        line.update(run_rusolorn(args))
+        line["value"] = line["rusolorn"]["decode_b8"]["tok_s"]
         line["seconds_total"] = round(time.perf_counter() - started, 1)
         print(json.dumps(line))
         return 0

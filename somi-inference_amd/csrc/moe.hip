@@ -24,22 +24,76 @@ __device__ __forceinline__ float clamped_glu(float g, float u, float limit, floa
     return g / (1.0f + expf(-alpha * g)) * (u + shift);
 }
 
-// One workgroup per token.
+// The router's logits for widths that are a multiple of 4: a workgroup owns ROUTE_TOKENS tokens and ROUTE_EXPERTS
+// experts (8 a wavefront); the tokens' x goes through LDS 256 channels at a time, a lane multiplies 4 channels of every
+// chunk, and a (token, expert) sum is the lanes' partial sums added by `wave_sum`: one order whatever else runs.
+#define ROUTE_TOKENS 8
+#define ROUTE_EXPERTS 32
+typedef __attribute__((ext_vector_type(4))) float route_f32x4;
+
 template <typename T>
 __global__ void __launch_bounds__(256)
-moe_route_kernel(const T* __restrict__ x, int64_t row_stride, const float* __restrict__ router, int width, int experts,
+moe_router_logits_kernel(const T* __restrict__ x, int64_t row_stride, const float* __restrict__ router, int n_tokens,
+                         int width, int experts, float* __restrict__ logits /*[N, experts]*/) {
+    __shared__ __attribute__((aligned(16))) float xs[ROUTE_TOKENS][256];
+    const int t0 = blockIdx.x * ROUTE_TOKENS;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int e0 = blockIdx.y * ROUTE_EXPERTS + wave * (ROUTE_EXPERTS / 4);
+    float acc[ROUTE_EXPERTS / 4][ROUTE_TOKENS];
+#pragma unroll
+    for (int ei = 0; ei < ROUTE_EXPERTS / 4; ++ei)
+#pragma unroll
+        for (int tt = 0; tt < ROUTE_TOKENS; ++tt) acc[ei][tt] = 0.f;
+    for (int k0 = 0; k0 < width; k0 += 256) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < ROUTE_TOKENS * 256; i += 256) {
+            const int tt = i >> 8, k = k0 + (i & 255);
+            xs[tt][i & 255] = (t0 + tt < n_tokens && k < width) ? to_float(x[(int64_t)(t0 + tt) * row_stride + k]) : 0.f;
+        }
+        __syncthreads();
+        const int k = k0 + lane * 4;
+        route_f32x4 xv[ROUTE_TOKENS];
+#pragma unroll
+        for (int tt = 0; tt < ROUTE_TOKENS; ++tt) xv[tt] = *reinterpret_cast<const route_f32x4*>(&xs[tt][lane * 4]);
+#pragma unroll
+        for (int ei = 0; ei < ROUTE_EXPERTS / 4; ++ei) {
+            route_f32x4 w = {0.f, 0.f, 0.f, 0.f};
+            if (e0 + ei < experts && k < width) w = *reinterpret_cast<const route_f32x4*>(router + (int64_t)(e0 + ei) * width + k);
+#pragma unroll
+            for (int tt = 0; tt < ROUTE_TOKENS; ++tt)
+                acc[ei][tt] += w[0] * xv[tt][0] + w[1] * xv[tt][1] + w[2] * xv[tt][2] + w[3] * xv[tt][3];
+        }
+    }
+#pragma unroll
+    for (int ei = 0; ei < ROUTE_EXPERTS / 4; ++ei)
+#pragma unroll
+        for (int tt = 0; tt < ROUTE_TOKENS; ++tt) {
+            const float total = wave_sum(acc[ei][tt]);
+            if (lane == 0 && e0 + ei < experts && t0 + tt < n_tokens) logits[(int64_t)(t0 + tt) * experts + e0 + ei] = total;
+        }
+}
+
+// One workgroup per token: the logits (given, or computed here for widths that are no multiple of 4), then the choice.
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const T* __restrict__ x, int64_t row_stride, const float* __restrict__ router,
+                 const float* __restrict__ logits, int width, int experts,
                  int top, int groups, int keep, int* __restrict__ chosen, float* __restrict__ weight) {
     __shared__ float score[MOE_MAX_EXPERTS];
     __shared__ int allowed[MOE_MAX_EXPERTS];
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const T* row = x + t * row_stride;
-    for (int e = wave; e < experts; e += 4) {
-        const float* w = router + (int64_t)e * width;
-        float acc = 0.f;
-        for (int i = lane; i < width; i += 64) acc += to_float(row[i]) * w[i];
-        acc = wave_sum(acc);
-        if (lane == 0) score[e] = acc;
+    if (logits != nullptr) {
+        for (int e = threadIdx.x; e < experts; e += 256) score[e] = logits[t * experts + e];
+    } else {
+        const T* row = x + t * row_stride;
+        for (int e = wave; e < experts; e += 4) {
+            const float* w = router + (int64_t)e * width;
+            float acc = 0.f;
+            for (int i = lane; i < width; i += 64) acc += to_float(row[i]) * w[i];
+            acc = wave_sum(acc);
+            if (lane == 0) score[e] = acc;
+        }
     }
     __syncthreads();
     if (threadIdx.x != 0) return;
@@ -95,23 +149,33 @@ moe_route_kernel(const T* __restrict__ x, int64_t row_stride, const float* __res
     }
 }
 
-extern "C" int somi_moe_route(const void* x, int dtype, int64_t row_stride, const float* router, int n_tokens, int width,
-                              int experts, int top, int groups, int keep, int* chosen, float* weight,
-                              hipStream_t stream) {
+extern "C" int somi_moe_route(const void* x, int dtype, int64_t row_stride, const float* router, float* logits,
+                              int n_tokens, int width, int experts, int top, int groups, int keep, int* chosen,
+                              float* weight, hipStream_t stream) {
     SOMI_REQUIRE(n_tokens >= 0 && width > 0 && experts > 0 && experts <= MOE_MAX_EXPERTS, "moe_route: %d experts, 1 to %d are supported",
                  experts, MOE_MAX_EXPERTS);
     SOMI_REQUIRE(groups >= 1 && experts % groups == 0 && keep >= 1 && keep <= groups, "moe_route: %d groups (keep %d) do not divide %d experts",
                  groups, keep, experts);
     SOMI_REQUIRE(top >= 1 && top <= MOE_MAX_TOP && top <= keep * (experts / groups), "moe_route: top %d does not fit the kept experts", top);
     if (n_tokens == 0) return 0;
+    SOMI_REQUIRE(dtype == SOMI_F32 || dtype == SOMI_BF16, "moe_route: unknown dtype %d", dtype);
+    // logits: a workspace [n_tokens, experts]; used where the tiled kernel applies (a width that is a multiple of 4)
+    const bool tiled = logits != nullptr && width % 4 == 0 && (uintptr_t)router % 16 == 0;
+    if (tiled) {
+        const dim3 grid(ceil_div(n_tokens, ROUTE_TOKENS), ceil_div(experts, ROUTE_EXPERTS));
+        if (dtype == SOMI_F32)
+            hipLaunchKernelGGL(moe_router_logits_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, row_stride, router,
+                               n_tokens, width, experts, logits);
+        else
+            hipLaunchKernelGGL(moe_router_logits_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)x, row_stride, router,
+                               n_tokens, width, experts, logits);
+    }
     if (dtype == SOMI_F32)
         hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, (const float*)x, row_stride, router,
-                           width, experts, top, groups, keep, chosen, weight);
-    else if (dtype == SOMI_BF16)
-        hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(n_tokens), dim3(256), 0, stream, (const bf16*)x, row_stride, router,
-                           width, experts, top, groups, keep, chosen, weight);
+                           tiled ? logits : nullptr, width, experts, top, groups, keep, chosen, weight);
     else
-        return somi_fail("moe_route: unknown dtype %d", dtype);
+        hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(n_tokens), dim3(256), 0, stream, (const bf16*)x, row_stride, router,
+                           tiled ? logits : nullptr, width, experts, top, groups, keep, chosen, weight);
     SOMI_LAUNCH_CHECK("moe_route");
     return 0;
 }
@@ -250,6 +314,129 @@ extern "C" int somi_moe_product(const void* a, int64_t a_stride, const void* w, 
     }
 #undef SOMI_MOE
     SOMI_LAUNCH_CHECK("moe_product");
+    return 0;
+}
+
+// The same products on the matrix cores (bfloat16, K a multiple of 8, rows aligned to 16 bytes): a workgroup owns one
+// row tile of up to 64 sorted rows and 4 x 64 output columns (GATED: 4 x 32 columns of gate and the same of up), a
+// wavefront up to four 16-row fragments (as many as the tile has rows for) against four 16-column fragments of `v_mfma_f32_16x16x32_bf16`.  Both operands have
+// K contiguous in memory, so a lane's fragment is one 16-byte load (rows of x by token, rows of W by output column);
+// the next K step's fragments are asked for before this step's products.  Sums run over K in one order per row.
+typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float moe_f32x4;
+#define MOE_MFMA_ROWS 64
+#define MOE_MFMA_FRAGS (MOE_MFMA_ROWS / 16)
+
+template <bool GATED>
+__global__ void __launch_bounds__(256)
+moe_product_mfma_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16* __restrict__ w,
+                        const int* __restrict__ tiles, const int* __restrict__ order,
+                        const float* __restrict__ pair_weight, int top, int n_out, int K, float limit, float alpha,
+                        float shift, void* __restrict__ out_) {
+    const int expert = tiles[blockIdx.x * 3];
+    if (expert < 0) return;
+    const int first = tiles[blockIdx.x * 3 + 1], rows = tiles[blockIdx.x * 3 + 2];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    constexpr int WAVE_COLS = GATED ? 32 : 64;           // output columns of a wavefront
+    const int col0 = (blockIdx.y * 4 + wave) * WAVE_COLS;
+    if (col0 >= n_out) return;
+    const bf16* wg = w + (int64_t)expert * (GATED ? 2 : 1) * n_out * K;
+    // this lane's rows of the two operands
+    const bf16* arow[MOE_MFMA_FRAGS];
+    bool alive[MOE_MFMA_FRAGS];
+#pragma unroll
+    for (int f = 0; f < MOE_MFMA_FRAGS; ++f) {
+        const int row = f * 16 + r;
+        alive[f] = row < rows;
+        const int64_t src = alive[f] ? (GATED ? (int64_t)(order[first + row] / top) : (int64_t)(first + row)) : 0;
+        arow[f] = a + src * a_stride + g * 8;
+    }
+    const bf16* brow[4];
+    bool blive[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        // GATED: fragments 0, 1 are gate columns col0 .. col0 + 31, fragments 2, 3 the up rows of the same columns
+        const int col = GATED ? col0 + (c & 1) * 16 + r : col0 + c * 16 + r;
+        blive[c] = col < n_out;
+        const int64_t wrow = GATED ? (int64_t)(c >> 1) * n_out + col : (int64_t)col;
+        brow[c] = wg + (blive[c] ? wrow : 0) * K + g * 8;
+    }
+    const int frags = (rows + 15) >> 4;               // the same for the whole workgroup
+    moe_f32x4 acc[MOE_MFMA_FRAGS][4];
+#pragma unroll
+    for (int f = 0; f < MOE_MFMA_FRAGS; ++f)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[f][c] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+    const moe_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    moe_bf16x8 fa[MOE_MFMA_FRAGS], fb[4], na[MOE_MFMA_FRAGS], nb[4];
+    auto fetch = [&](moe_bf16x8 (&xa)[MOE_MFMA_FRAGS], moe_bf16x8 (&xb)[4], int k0) {
+        const bool inside = k0 + g * 8 < K;
+#pragma unroll
+        for (int f = 0; f < MOE_MFMA_FRAGS; ++f)
+            xa[f] = (inside && alive[f]) ? *reinterpret_cast<const moe_bf16x8*>(arow[f] + k0) : zero;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            xb[c] = (inside && blive[c]) ? *reinterpret_cast<const moe_bf16x8*>(brow[c] + k0) : zero;
+    };
+    fetch(fa, fb, 0);
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        if (k0 + 32 < K) fetch(na, nb, k0 + 32);
+#pragma unroll
+        for (int f = 0; f < MOE_MFMA_FRAGS; ++f)
+            if (f < frags) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    acc[f][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[f], fb[c], acc[f][c], 0, 0, 0);
+            }
+#pragma unroll
+        for (int f = 0; f < MOE_MFMA_FRAGS; ++f) fa[f] = na[f];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) fb[c] = nb[c];
+    }
+    // a lane holds rows g * 4 + i of a fragment's 16 and column r of its 16
+#pragma unroll
+    for (int f = 0; f < MOE_MFMA_FRAGS; ++f)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = f * 16 + g * 4 + i;
+            if (row >= rows) continue;
+            if (GATED) {
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const int col = col0 + c * 16 + r;
+                    if (col < n_out)
+                        ((bf16*)out_)[(int64_t)(first + row) * n_out + col] =
+                            (bf16)clamped_glu(acc[f][c][i], acc[f][c + 2][i], limit, alpha, shift);
+                }
+            } else {
+                const int pair = order[first + row];
+                const float pw = pair_weight[pair];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int col = col0 + c * 16 + r;
+                    if (col < n_out) ((float*)out_)[(int64_t)pair * n_out + col] = pw * acc[f][c][i];
+                }
+            }
+        }
+}
+
+extern "C" int somi_moe_product_mfma(const void* a, int64_t a_stride, const void* w, int gated, const int* tiles,
+                                     int max_tiles, const int* order, const float* pair_weight, int top, int n_out, int K,
+                                     float limit, float alpha, float shift, void* out, hipStream_t stream) {
+    SOMI_REQUIRE(max_tiles >= 0 && n_out > 0 && K > 0 && top > 0 && a_stride >= K, "moe_product_mfma: bad sizes");
+    SOMI_REQUIRE(K % 8 == 0 && a_stride % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0,
+                 "moe_product_mfma: K of %d or rows that are not aligned to 16 bytes", K);
+    if (max_tiles == 0) return 0;
+    const dim3 grid(max_tiles, ceil_div(n_out, gated ? 128 : 256));
+    SOMI_REQUIRE(grid.y <= 65535, "moe_product_mfma: too many columns");
+    if (gated)
+        hipLaunchKernelGGL(moe_product_mfma_kernel<true>, grid, dim3(256), 0, stream, (const bf16*)a, a_stride, (const bf16*)w,
+                           tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
+    else
+        hipLaunchKernelGGL(moe_product_mfma_kernel<false>, grid, dim3(256), 0, stream, (const bf16*)a, a_stride, (const bf16*)w,
+                           tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
+    SOMI_LAUNCH_CHECK("moe_product_mfma");
     return 0;
 }
 

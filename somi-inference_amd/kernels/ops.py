@@ -1062,9 +1062,10 @@ def delta_prepare(rows: torch.Tensor, ab: torch.Tensor, taps: torch.Tensor, conv
 
 
 def delta_scan(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, entry_start: torch.Tensor,
-               state_slots: torch.Tensor, state: torch.Tensor, groups: int) -> torch.Tensor:
+               state_slots: torch.Tensor, state: torch.Tensor, groups: int, lanes: int = 0) -> torch.Tensor:
     """The recurrence S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q per head over every entry's tokens, from
-    and into ``state[state_slots[e]]`` ([slots, heads, dim, vdim] float32) -> o [N, heads, vdim] float32."""
+    and into ``state[state_slots[e]]`` ([slots, heads, dim, vdim] float32) -> o [N, heads, vdim] float32.  ``lanes``: lanes that
+    share a column of the state (4 or 16; 0: the launcher chooses by the model's sizes and the device)."""
     _need(state, "recurrent state", torch.float32)
     _, heads, dim, vdim = state.shape
     n = qkv.shape[0]
@@ -1076,12 +1077,20 @@ def delta_scan(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, entry
     _need(state_slots, "state slots", torch.int32, (entries,))
     o = torch.empty((n, heads, vdim), dtype=torch.float32, device=qkv.device)
     _check(library().somi_delta_scan(_ptr(qkv), _ptr(beta), _ptr(decay), _ptr(entry_start), _ptr(state_slots), _ptr(state),
-                                     entries, groups, heads, dim, vdim, _ptr(o), _stream()))
+                                     entries, groups, heads, dim, vdim, int(lanes), _ptr(o), _stream()))
     return o
 
 
 # ------------------------------------------------------------------------------------------ mixture of experts
-MOE_TILE_ROWS = 16
+MOE_TILE_ROWS = 16           # sorted rows of a tile of the plain products
+MOE_MFMA_ROWS = 64           # ... and of the matrix-core products
+
+
+def moe_mfma_supported(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor) -> bool:
+    """The matrix-core products take these operands: bfloat16, both K (the width and the experts' size) multiples of 8,
+    rows aligned to 16 bytes."""
+    return (x.dtype == torch.bfloat16 and gate_up.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and down.shape[2] % 8 == 0
+            and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and gate_up.data_ptr() % 16 == 0 and down.data_ptr() % 16 == 0)
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, top: int, groups: int, keep: int) -> tuple[torch.Tensor, torch.Tensor]:
@@ -1094,27 +1103,29 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, top: int, groups: int, keep
         raise KernelError(f"moe_route: router {tuple(router.shape)} does not fit rows of {width}")
     chosen = torch.empty((n, top), dtype=torch.int32, device=x.device)
     weight = torch.empty((n, top), dtype=torch.float32, device=x.device)
-    _check(library().somi_moe_route(_ptr(x), dtype_code(x.dtype), ctypes.c_int64(x.stride(0)), _ptr(router), n, width,
-                                    router.shape[0], int(top), int(groups), int(keep), _ptr(chosen), _ptr(weight), _stream()))
+    logits = torch.empty((n, router.shape[0]), dtype=torch.float32, device=x.device)     # the router's sums, if it tiles them
+    _check(library().somi_moe_route(_ptr(x), dtype_code(x.dtype), ctypes.c_int64(x.stride(0)), _ptr(router), _ptr(logits), n,
+                                    width, router.shape[0], int(top), int(groups), int(keep), _ptr(chosen), _ptr(weight),
+                                    _stream()))
     return chosen, weight
 
 
-def moe_align(chosen: torch.Tensor, experts: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+def moe_align(chosen: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """The (token, expert) pairs sorted by expert: (order [pairs] int32, offsets [experts + 1] int32, tiles [T, 3] int32
-    = (expert or -1, first sorted row, rows) for row tiles of MOE_TILE_ROWS)."""
+    = (expert or -1, first sorted row, rows) for row tiles of ``tile_rows``)."""
     _need(chosen, "chosen experts", torch.int32)
     pairs = chosen.numel()
-    max_tiles = library().somi_moe_max_tiles(pairs, int(experts), MOE_TILE_ROWS)
+    max_tiles = library().somi_moe_max_tiles(pairs, int(experts), int(tile_rows))
     order = torch.empty((pairs,), dtype=torch.int32, device=chosen.device)
     offsets = torch.empty((experts + 1,), dtype=torch.int32, device=chosen.device)
     tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=chosen.device)
-    _check(library().somi_moe_align(_ptr(chosen), pairs, int(experts), MOE_TILE_ROWS, max_tiles, _ptr(order), _ptr(offsets),
+    _check(library().somi_moe_align(_ptr(chosen), pairs, int(experts), int(tile_rows), max_tiles, _ptr(order), _ptr(offsets),
                                     _ptr(tiles), _stream()))
     return order, offsets, tiles
 
 
 def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, top: int,
-                limit: float, alpha: float, shift: float) -> torch.Tensor:
+                limit: float, alpha: float, shift: float, mfma: bool = False) -> torch.Tensor:
     """act[p] = glu(W_gate[e] x[t], W_up[e] x[t]) for the sorted pairs p = (t, e); gate_up: [experts, 2 F, K], gate rows
     first -> [pairs, F]."""
     _need(x, "rows")
@@ -1124,6 +1135,11 @@ def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, tiles: torch.Tensor, ord
         raise KernelError(f"moe_gate_up: matrices {tuple(gate_up.shape)} do not fit rows of {x.shape[1]}")
     pairs = order.numel()
     act = torch.empty((pairs, two_f // 2), dtype=x.dtype, device=x.device)
+    if mfma:
+        _check(library().somi_moe_product_mfma(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(gate_up), 1, _ptr(tiles), tiles.shape[0],
+                                               _ptr(order), None, int(top), two_f // 2, k, ctypes.c_float(limit),
+                                               ctypes.c_float(alpha), ctypes.c_float(shift), _ptr(act), _stream()))
+        return act
     _check(library().somi_moe_product(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(gate_up), dtype_code(x.dtype), 1, _ptr(tiles),
                                       tiles.shape[0], _ptr(order), None, int(top), two_f // 2, k, ctypes.c_float(limit),
                                       ctypes.c_float(alpha), ctypes.c_float(shift), _ptr(act), _stream()))
@@ -1131,7 +1147,7 @@ def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, tiles: torch.Tensor, ord
 
 
 def moe_down(act: torch.Tensor, down: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, weight: torch.Tensor,
-             top: int) -> torch.Tensor:
+             top: int, mfma: bool = False) -> torch.Tensor:
     """y[pair] = weight[pair] * W_down[e] act[p] -> [pairs, width] float32, at the pairs' own places."""
     _need(act, "activations")
     _need(down, "down matrices", act.dtype)
@@ -1140,6 +1156,11 @@ def moe_down(act: torch.Tensor, down: torch.Tensor, tiles: torch.Tensor, order: 
         raise KernelError(f"moe_down: matrices {tuple(down.shape)} do not fit activations of {act.shape[1]}")
     _need(weight, "pair weights", torch.float32)
     y = torch.empty((order.numel(), width), dtype=torch.float32, device=act.device)
+    if mfma:
+        _check(library().somi_moe_product_mfma(_ptr(act), ctypes.c_int64(act.stride(0)), _ptr(down), 0, _ptr(tiles), tiles.shape[0],
+                                               _ptr(order), _ptr(weight), int(top), width, k, ctypes.c_float(0.0),
+                                               ctypes.c_float(0.0), ctypes.c_float(0.0), _ptr(y), _stream()))
+        return y
     _check(library().somi_moe_product(_ptr(act), ctypes.c_int64(act.stride(0)), _ptr(down), dtype_code(act.dtype), 0, _ptr(tiles),
                                       tiles.shape[0], _ptr(order), _ptr(weight), int(top), width, k, ctypes.c_float(0.0),
                                       ctypes.c_float(0.0), ctypes.c_float(0.0), _ptr(y), _stream()))

@@ -206,6 +206,35 @@ def test_gated_delta_rule_against_the_plain_function(dtype, heads, groups, dim, 
             torch.testing.assert_close(cut, want, **tol(dtype, loose=4))
 
 
+@pytest.mark.parametrize("lanes", [4, 16])
+@pytest.mark.parametrize("heads,groups,dim,vdim", [(2, 1, 16, 32), (3, 3, 20, 24), (2, 2, 128, 16), (1, 1, 200, 40), (2, 1, 64, 130)])
+def test_the_recurrence_with_either_number_of_lanes_a_column(lanes, heads, groups, dim, vdim):
+    """The kernel of the recurrence alone, from a state that is not zero, with 4 and with 16 lanes a column."""
+    gen = torch.Generator().manual_seed(dim + lanes)
+    tokens, channels = 45, 2 * groups * dim + heads * vdim
+    qkv = torch.randn(tokens, channels, generator=gen)
+    qkv[:, :2 * groups * dim] = torch.nn.functional.normalize(qkv[:, :2 * groups * dim].view(tokens, 2 * groups, dim), dim=-1).view(tokens, -1)
+    beta, decay = torch.rand(tokens, heads, generator=gen), 0.5 + 0.5 * torch.rand(tokens, heads, generator=gen)
+    state = torch.randn(3, heads, dim, vdim, generator=gen)
+    want_state, want = state.clone(), torch.zeros(tokens, heads, vdim)
+    cuts = [0, 7, 45]                                      # two entries: slot 2 takes tokens 0..6, slot 0 the rest
+    for (lo, hi), slot in zip(zip(cuts, cuts[1:]), (2, 0)):
+        for t in range(lo, hi):
+            for a in range(heads):
+                g = a // (heads // groups)
+                q, k = qkv[t, g * dim:(g + 1) * dim], qkv[t, (groups + g) * dim:(groups + g + 1) * dim]
+                v = qkv[t, 2 * groups * dim + a * vdim:2 * groups * dim + (a + 1) * vdim]
+                S = decay[t, a] * want_state[slot, a]
+                S = S + torch.outer(k, beta[t, a] * (v - S.T @ k))
+                want_state[slot, a], want[t, a] = S, S.T @ q
+    on_device = state.to(DEV)
+    got = ops.delta_scan(qkv.to(DEV), beta.to(DEV), decay.to(DEV), torch.tensor(cuts, dtype=torch.int32, device=DEV),
+                         torch.tensor([2, 0], dtype=torch.int32, device=DEV), on_device, groups, lanes=lanes)
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(on_device.cpu(), want_state, rtol=1e-4, atol=1e-4)
+    assert torch.equal(on_device[1].cpu(), state[1])              # a slot of no entry is left alone
+
+
 def test_two_requests_side_by_side_keep_their_own_state():
     part = delta_part(32, 2, 1, 16, 16, 3)
     weights = random_weights(part, torch.float32, seed=9)
