@@ -73,21 +73,38 @@ moe_router_logits_kernel(const T* __restrict__ x, int64_t row_stride, const floa
         }
 }
 
-// One workgroup per token: the logits (given, or computed here for widths that are no multiple of 4), then the choice.
+// The choice, one wavefront per token: the logits (given, or computed here for widths that are no multiple of 4), the
+// softmax, the best runs, the best experts of those.  A lane owns the experts lane, lane + 64, ...; the best of all
+// lanes' candidates is found by exchanging (score, index) pairs, ties to the lower index.
+__device__ __forceinline__ void wave_best(float& value, int& index) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float other = __shfl_xor(value, off, 64);
+        const int other_index = __shfl_xor(index, off, 64);
+        if (other > value || (other == value && other_index < index)) {
+            value = other;
+            index = other_index;
+        }
+    }
+}
+
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64)
 moe_route_kernel(const T* __restrict__ x, int64_t row_stride, const float* __restrict__ router,
                  const float* __restrict__ logits, int width, int experts,
                  int top, int groups, int keep, int* __restrict__ chosen, float* __restrict__ weight) {
+    constexpr int PER_LANE = MOE_MAX_EXPERTS / 64;
     __shared__ float score[MOE_MAX_EXPERTS];
-    __shared__ int allowed[MOE_MAX_EXPERTS];
+    __shared__ int taken[MOE_MAX_EXPERTS];          // per run: kept or not
+    __shared__ float pick_score[MOE_MAX_TOP];
+    __shared__ int pick_index[MOE_MAX_TOP];
     const int64_t t = blockIdx.x;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int lane = threadIdx.x;
     if (logits != nullptr) {
-        for (int e = threadIdx.x; e < experts; e += 256) score[e] = logits[t * experts + e];
+        for (int e = lane; e < experts; e += 64) score[e] = logits[t * experts + e];
     } else {
         const T* row = x + t * row_stride;
-        for (int e = wave; e < experts; e += 4) {
+        for (int e = 0; e < experts; ++e) {
             const float* w = router + (int64_t)e * width;
             float acc = 0.f;
             for (int i = lane; i < width; i += 64) acc += to_float(row[i]) * w[i];
@@ -96,56 +113,96 @@ moe_route_kernel(const T* __restrict__ x, int64_t row_stride, const float* __res
         }
     }
     __syncthreads();
-    if (threadIdx.x != 0) return;
-    float top_z = score[0];
-    for (int e = 1; e < experts; ++e) top_z = fmaxf(top_z, score[e]);
+    float s[PER_LANE];
+    float top_z = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+        const int e = lane + 64 * j;
+        s[j] = e < experts ? score[e] : -INFINITY;
+        top_z = fmaxf(top_z, s[j]);
+    }
+    top_z = wave_max(top_z);
     float total = 0.f;
-    for (int e = 0; e < experts; ++e) {
-        score[e] = expf(score[e] - top_z);
-        total += score[e];
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+        s[j] = lane + 64 * j < experts ? expf(s[j] - top_z) : 0.f;
+        total += s[j];
     }
-    for (int e = 0; e < experts; ++e) {
-        score[e] /= total;
-        allowed[e] = 0;
+    total = wave_sum(total);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+        s[j] /= total;
+        if (lane + 64 * j < experts) score[lane + 64 * j] = s[j];
     }
+    for (int g = lane; g < groups; g += 64) taken[g] = keep >= groups ? 1 : 0;
+    __syncthreads();
     const int per = experts / groups;
-    // the keep best runs, one at a time (a run already taken is marked through its first expert's flag)
-    for (int round = 0; round < keep; ++round) {
-        int best = -1;
-        float best_score = -1.f;
-        for (int g = 0; g < groups; ++g) {
-            if (allowed[g * per]) continue;
-            float s = score[g * per];
-            for (int j = 1; j < per; ++j) s = fmaxf(s, score[g * per + j]);
-            if (s > best_score) {
-                best_score = s;
-                best = g;
+    if (keep < groups) {
+        // a lane owns the runs lane, lane + 64, ...: their scores, then `keep` rounds of the best run not yet kept
+        float run[PER_LANE];
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) {
+            const int g = lane + 64 * j;
+            run[j] = -1.f;
+            if (g < groups) {
+                run[j] = score[g * per];
+                for (int i = 1; i < per; ++i) run[j] = fmaxf(run[j], score[g * per + i]);
             }
         }
-        if (best < 0) break;
-        for (int j = 0; j < per; ++j) allowed[best * per + j] = 1;
+        for (int round = 0; round < keep; ++round) {
+            float best = -1.f;
+            int best_run = 1 << 30;
+#pragma unroll
+            for (int j = 0; j < PER_LANE; ++j)
+                if (run[j] > best) {
+                    best = run[j];
+                    best_run = lane + 64 * j;
+                }
+            wave_best(best, best_run);
+            if (best_run >= groups) break;                 // nothing left that compares (scores that are not numbers)
+#pragma unroll
+            for (int j = 0; j < PER_LANE; ++j)
+                if (lane + 64 * j == best_run) {
+                    run[j] = -1.f;
+                    taken[best_run] = 1;
+                }
+        }
+        __syncthreads();
     }
-    int picks[MOE_MAX_TOP];
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+        const int e = lane + 64 * j;
+        if (e >= experts || !taken[e / per]) s[j] = -1.f;  // out of the choice
+    }
     float sum = 0.f;
-    for (int j = 0; j < top; ++j) {
-        int best = -1;
-        float best_score = -1.f;
-        for (int e = 0; e < experts; ++e)
-            if (allowed[e] == 1 && score[e] > best_score) {
-                best_score = score[e];
-                best = e;
+    for (int pick = 0; pick < top; ++pick) {
+        float best = -1.f;
+        int best_expert = 1 << 30;
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j)
+            if (s[j] > best) {
+                best = s[j];
+                best_expert = lane + 64 * j;
             }
-        if (best < 0) {          // scores that compare with nothing (not a number): any expert, weight as it comes
-            best = 0;
-            best_score = score[0];
+        wave_best(best, best_expert);
+        if (best_expert >= experts) {                      // scores that compare with nothing: any expert, weight as it comes
+            best_expert = 0;
+            best = score[0];
         }
-        picks[j] = best;
-        allowed[best] = 2;
-        sum += best_score;
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j)
+            if (lane + 64 * j == best_expert) s[j] = -1.f;
+        if (lane == 0) {
+            pick_score[pick] = best;
+            pick_index[pick] = best_expert;
+        }
+        sum += best;
     }
-    for (int j = 0; j < top; ++j) {
-        chosen[t * top + j] = picks[j];
-        weight[t * top + j] = score[picks[j]] / (sum + 1e-20f);
+    __syncthreads();
+    for (int pick = lane; pick < top; pick += 64) {
+        chosen[t * top + pick] = pick_index[pick];
+        weight[t * top + pick] = pick_score[pick] / (sum + 1e-20f);
     }
 }
 
@@ -171,10 +228,10 @@ extern "C" int somi_moe_route(const void* x, int dtype, int64_t row_stride, cons
                                n_tokens, width, experts, logits);
     }
     if (dtype == SOMI_F32)
-        hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, (const float*)x, row_stride, router,
+        hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n_tokens), dim3(64), 0, stream, (const float*)x, row_stride, router,
                            tiled ? logits : nullptr, width, experts, top, groups, keep, chosen, weight);
     else
-        hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(n_tokens), dim3(256), 0, stream, (const bf16*)x, row_stride, router,
+        hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(n_tokens), dim3(64), 0, stream, (const bf16*)x, row_stride, router,
                            tiled ? logits : nullptr, width, experts, top, groups, keep, chosen, weight);
     SOMI_LAUNCH_CHECK("moe_route");
     return 0;

@@ -30,7 +30,7 @@ RUSOLORN = {
         vocab=211, width=96, norm_eps=1e-5, embedding_scale=4.0, residual_mult=0.5, token_side_dim=8, layers=(
             layer((4, 2, 16, 24, 0.5), (4, 2, 16, 32, 4),
                   dict(experts=8, top=2, ff=48, limit=1.0, groups=4, keep=2, shared_ff=64, shared_limit=2.5)),
-            layer((6, 1, 32, 40, 0.3), (2, 1, 32, 16, 3),
+            layer((6, 1, 32, 36, 0.3), (2, 1, 32, 16, 3),
                   dict(experts=6, top=3, ff=32, limit=2.0, groups=3, keep=2, shared_ff=16, shared_limit=0.5)),
             layer((4, 2, 16, 24, 0.5), (4, 2, 16, 32, 4),
                   dict(experts=8, top=2, ff=48, limit=1.0, groups=4, keep=2, shared_ff=64, shared_limit=2.5)),

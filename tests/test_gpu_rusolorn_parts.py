@@ -119,7 +119,7 @@ def attention_part(width, heads, groups, dim, window, scale, eps=1e-5):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,groups,dim,window,page,tokens", [(4, 2, 16, 24, 16, 150), (3, 3, 24, 1000, 8, 70),
-                                                               (6, 1, 48, 40, 16, 300), (2, 1, 20, 1, 4, 30),
+                                                               (6, 2, 48, 56, 16, 300), (2, 1, 20, 1, 4, 30),
                                                                (2, 2, 64, 7, 8, 90)])
 def test_tied_value_attention_against_the_plain_function(dtype, heads, groups, dim, window, page, tokens):
     width = 64
@@ -142,7 +142,7 @@ def test_tied_value_attention_against_the_plain_function(dtype, heads, groups, d
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("window,page", [(40, 16), (33, 8), (9, 4), (16, 16), (1, 8)])
+@pytest.mark.parametrize("window,page", [(44, 16), (33, 8), (9, 4), (16, 16), (1, 8)])
 @pytest.mark.parametrize("decoded", [False, True])
 def test_one_key_stands_out_exactly_inside_the_window(dtype, window, page, decoded):
     """The query and key projections pick disjoint channels of the input, so queries and keys are set at will: one key

@@ -52,7 +52,7 @@ def test_replay_of_a_rusolorn_folder(dtype, tmp_path):
         want[rid] = plain.forward(config, weights, tokens, margins=margins)
         close[rid] = set((torch.stack(margins).min(dim=0).values < CLOSE_CALL).nonzero().flatten().tolist())
 
-    # most of a request in one step, its last 40 tokens one by one (they pass the windows of 24 and 40 tokens)
+    # most of a request in one step, its last 40 tokens one by one (they pass the windows of 24 and 36 tokens)
     b = requests["e"]
     steps, expect = [{"step": 0, "entries": [{"id": "dec", "tokens": b[:-40], "want": [0, len(b) - 41]}], "end": []}], {}
     expect[0] = want["e"][[0, len(b) - 41]]
