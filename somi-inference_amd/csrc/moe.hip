@@ -478,16 +478,147 @@ moe_product_mfma_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16
         }
 }
 
+// The same for experts with many rows (prompt portions): a row tile of up to 128 sorted rows x 256 columns.  The rows'
+// part of a round of four K steps (128 rows x 128 values) goes through LDS, loaded once by the workgroup (rows padded by 16
+// bytes against bank conflicts), two buffers, one barrier a round; every wavefront reads all eight row fragments from LDS
+// and its own four column fragments of the weights straight from memory, a round (128 matrix instructions) ahead.  A weight fragment now serves eight row fragments instead of four, and the rows are read from memory once
+// instead of once a wavefront.
+#define MOE_BIG_ROWS 128
+#define MOE_BIG_FRAGS (MOE_BIG_ROWS / 16)
+#define MOE_BIG_KS 4                                        // K steps of 32 that one round of loads brings
+#define MOE_BIG_ROW_BYTES (MOE_BIG_KS * 64 + 16)            // a row's part of a round in LDS, padded against bank conflicts
+#define MOE_BIG_PIECES (MOE_BIG_ROWS * MOE_BIG_KS * 4 / 256) // 16-byte pieces of the rows a thread stages a round
+
+template <bool GATED>
+__global__ void __launch_bounds__(256)
+moe_product_mfma_big_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16* __restrict__ w,
+                            const int* __restrict__ tiles, const int* __restrict__ order,
+                            const float* __restrict__ pair_weight, int top, int n_out, int K, float limit, float alpha,
+                            float shift, void* __restrict__ out_) {
+    __shared__ __attribute__((aligned(16))) char rows_lds[2][MOE_BIG_ROWS * MOE_BIG_ROW_BYTES];
+    const int expert = tiles[blockIdx.x * 3];
+    if (expert < 0) return;
+    const int first = tiles[blockIdx.x * 3 + 1], rows = tiles[blockIdx.x * 3 + 2];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 15, g = lane >> 4;
+    constexpr int WAVE_COLS = GATED ? 32 : 64;
+    constexpr int ROUND = MOE_BIG_KS * 32;                      // K values of a round
+    constexpr int PPR = MOE_BIG_KS * 4;                         // 16-byte pieces of a row in a round
+    const int col0 = (blockIdx.y * 4 + wave) * WAVE_COLS;      // may lie past n_out: the wavefront then only helps to stage
+    const bf16* wg = w + (int64_t)expert * (GATED ? 2 : 1) * n_out * K;
+    // the pieces of the rows' round that this thread stages: piece p = tid + 256 j is piece p % PPR of row p / PPR
+    const bf16* srow[MOE_BIG_PIECES];
+    int sk[MOE_BIG_PIECES], slds[MOE_BIG_PIECES];
+#pragma unroll
+    for (int j = 0; j < MOE_BIG_PIECES; ++j) {
+        const int p = tid + 256 * j, row = p / PPR, piece = p % PPR;
+        const bool live = row < rows;
+        const int64_t src = live ? (GATED ? (int64_t)(order[first + row] / top) : (int64_t)(first + row)) : 0;
+        srow[j] = a + src * a_stride + piece * 8;
+        sk[j] = live ? piece * 8 : K;                            // a dead row's pieces count as past K: zeros
+        slds[j] = row * MOE_BIG_ROW_BYTES + piece * 16;
+    }
+    const bf16* brow[4];
+    bool blive[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int col = GATED ? col0 + (c & 1) * 16 + r : col0 + c * 16 + r;
+        blive[c] = col < n_out;
+        const int64_t wrow = GATED ? (int64_t)(c >> 1) * n_out + col : (int64_t)col;
+        brow[c] = wg + (blive[c] ? wrow : 0) * K + g * 8;
+    }
+    const int frags = (rows + 15) >> 4;
+    moe_f32x4 acc[MOE_BIG_FRAGS][4];
+#pragma unroll
+    for (int f = 0; f < MOE_BIG_FRAGS; ++f)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[f][c] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+    const moe_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    moe_bf16x8 sa[MOE_BIG_PIECES], fb[MOE_BIG_KS][4], nb[MOE_BIG_KS][4];
+    auto fetch = [&](moe_bf16x8 (&xa)[MOE_BIG_PIECES], moe_bf16x8 (&xb)[MOE_BIG_KS][4], int k0) {
+#pragma unroll
+        for (int j = 0; j < MOE_BIG_PIECES; ++j)
+            xa[j] = k0 + sk[j] < K ? *reinterpret_cast<const moe_bf16x8*>(srow[j] + k0) : zero;
+#pragma unroll
+        for (int s = 0; s < MOE_BIG_KS; ++s) {
+            const bool inside = k0 + s * 32 + g * 8 < K;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                xb[s][c] = (inside && blive[c]) ? *reinterpret_cast<const moe_bf16x8*>(brow[c] + k0 + s * 32) : zero;
+        }
+    };
+    fetch(sa, fb, 0);
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += ROUND, buf ^= 1) {
+#pragma unroll
+        for (int j = 0; j < MOE_BIG_PIECES; ++j) *reinterpret_cast<moe_bf16x8*>(rows_lds[buf] + slds[j]) = sa[j];
+        __syncthreads();
+        if (k0 + ROUND < K) fetch(sa, nb, k0 + ROUND);
+#pragma unroll
+        for (int s = 0; s < MOE_BIG_KS; ++s) {
+            if (k0 + s * 32 >= K) break;
+#pragma unroll
+            for (int f = 0; f < MOE_BIG_FRAGS; ++f)
+                if (f < frags) {
+                    const moe_bf16x8 fa = *reinterpret_cast<const moe_bf16x8*>(
+                        rows_lds[buf] + (f * 16 + r) * MOE_BIG_ROW_BYTES + s * 64 + g * 16);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        acc[f][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, fb[s][c], acc[f][c], 0, 0, 0);
+                }
+        }
+#pragma unroll
+        for (int s = 0; s < MOE_BIG_KS; ++s)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) fb[s][c] = nb[s][c];
+    }
+    if (col0 >= n_out) return;
+#pragma unroll
+    for (int f = 0; f < MOE_BIG_FRAGS; ++f)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = f * 16 + g * 4 + i;
+            if (row >= rows) continue;
+            if (GATED) {
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const int col = col0 + c * 16 + r;
+                    if (col < n_out)
+                        ((bf16*)out_)[(int64_t)(first + row) * n_out + col] =
+                            (bf16)clamped_glu(acc[f][c][i], acc[f][c + 2][i], limit, alpha, shift);
+                }
+            } else {
+                const int pair = order[first + row];
+                const float pw = pair_weight[pair];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int col = col0 + c * 16 + r;
+                    if (col < n_out) ((float*)out_)[(int64_t)pair * n_out + col] = pw * acc[f][c][i];
+                }
+            }
+        }
+}
+
 extern "C" int somi_moe_product_mfma(const void* a, int64_t a_stride, const void* w, int gated, const int* tiles,
-                                     int max_tiles, const int* order, const float* pair_weight, int top, int n_out, int K,
-                                     float limit, float alpha, float shift, void* out, hipStream_t stream) {
+                                     int max_tiles, int tile_rows, const int* order, const float* pair_weight, int top,
+                                     int n_out, int K, float limit, float alpha, float shift, void* out,
+                                     hipStream_t stream) {
+    SOMI_REQUIRE(tile_rows == MOE_MFMA_ROWS || tile_rows == MOE_BIG_ROWS, "moe_product_mfma: tiles of %d rows (%d or %d)",
+                 tile_rows, MOE_MFMA_ROWS, MOE_BIG_ROWS);
     SOMI_REQUIRE(max_tiles >= 0 && n_out > 0 && K > 0 && top > 0 && a_stride >= K, "moe_product_mfma: bad sizes");
     SOMI_REQUIRE(K % 8 == 0 && a_stride % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0,
                  "moe_product_mfma: K of %d or rows that are not aligned to 16 bytes", K);
     if (max_tiles == 0) return 0;
     const dim3 grid(max_tiles, ceil_div(n_out, gated ? 128 : 256));
     SOMI_REQUIRE(grid.y <= 65535, "moe_product_mfma: too many columns");
-    if (gated)
+    if (tile_rows == MOE_BIG_ROWS) {
+        if (gated)
+            hipLaunchKernelGGL(moe_product_mfma_big_kernel<true>, grid, dim3(256), 0, stream, (const bf16*)a, a_stride,
+                               (const bf16*)w, tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
+        else
+            hipLaunchKernelGGL(moe_product_mfma_big_kernel<false>, grid, dim3(256), 0, stream, (const bf16*)a, a_stride,
+                               (const bf16*)w, tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
+    } else if (gated)
         hipLaunchKernelGGL(moe_product_mfma_kernel<true>, grid, dim3(256), 0, stream, (const bf16*)a, a_stride, (const bf16*)w,
                            tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
     else

@@ -105,13 +105,14 @@ class RoutedExperts(FeedForward):
             x = x.materialize()
         with stage("router"):
             chosen, weight = ops.moe_route(x, self.router, self.top, self.groups, self.keep_groups)
-            mfma = ops.moe_mfma_supported(x, self.gate_up, self.down)     # bfloat16: the products run on the matrix cores
-            order, _, tiles = ops.moe_align(chosen, self.num_experts, ops.MOE_MFMA_ROWS if mfma else ops.MOE_TILE_ROWS)
+            # bfloat16: the products run on the matrix cores, in tiles sized by the rows an expert gets in this step
+            rows = ops.moe_tile_rows(chosen.numel(), self.num_experts, ops.moe_mfma_supported(x, self.gate_up, self.down))
+            order, _, tiles = ops.moe_align(chosen, self.num_experts, rows)
         with stage("experts gate_up"):
             act = ops.moe_gate_up(x, self.gate_up, tiles, order, self.top, self.unit.limit, self.unit.alpha, self.unit.shift,
-                                  mfma=mfma)
+                                  tile_rows=rows)
         with stage("experts down"):
-            pairs = ops.moe_down(act, self.down, tiles, order, weight, self.top, mfma=mfma)
+            pairs = ops.moe_down(act, self.down, tiles, order, weight, self.top, tile_rows=rows)
         shared = None
         if self.shared_size:
             unit = self.shared_unit

@@ -60,7 +60,7 @@ def short_convolution(x: torch.Tensor, taps: torch.Tensor) -> torch.Tensor:
     """y[t, c] = sum_d taps[c, last - d] x[t - d, c] with zeros before the start, then SiLU."""
     tokens, width = x.shape[0], taps.shape[1]
     y = torch.zeros_like(x)
-    for d in range(width):
+    for d in range(min(width, tokens)):
         y[d:] += x[:tokens - d] * taps[:, width - 1 - d]
     return silu(y)
 

@@ -25,6 +25,8 @@ def layer(left, right, mlp=None) -> RusolornLayer:
 #    shared expert, no token input, multipliers of 1.
 # C: windows of one and of seven tokens, no convolution (one tap), large recurrent heads, every expert chosen,
 #    pages of 8 tokens, a width that is no multiple of 32.
+# D: a width that is no multiple of 8, odd sizes everywhere, five taps, three q/k-sharing recurrent heads, experts
+#    without groups beside a shared one, layers that differ in everything.
 RUSOLORN = {
     "A": dict(block_size=16, seed=5, config=RusolornConfig(
         vocab=211, width=96, norm_eps=1e-5, embedding_scale=4.0, residual_mult=0.5, token_side_dim=8, layers=(
@@ -45,6 +47,12 @@ RUSOLORN = {
             layer((2, 2, 48, 1, 0.2), (2, 1, 64, 128, 1), dict(experts=4, top=4, ff=24, limit=1.5, groups=2, keep=2)),
             layer((2, 1, 16, 7, 0.6), (2, 2, 8, 8, 1),
                   dict(experts=4, top=2, ff=24, limit=1.5, groups=4, keep=3, shared_ff=8, shared_limit=1.0)),
+        ))),
+    "D": dict(block_size=16, seed=8, config=RusolornConfig(
+        vocab=77, width=100, norm_eps=1e-5, embedding_scale=2.5, residual_mult=0.8, token_side_dim=7, layers=(
+            layer((5, 5, 12, 5, 0.7), (3, 1, 36, 28, 5), dict(experts=3, top=2, ff=20, limit=2.0, shared_ff=12, shared_limit=3.0)),
+            layer((1, 1, 40, 50, 0.3), (1, 1, 10, 6, 2), None),
+            layer((4, 2, 8, 9, 0.9), (6, 2, 6, 10, 3), dict(experts=7, top=3, ff=9, limit=0.7)),
         ))),
 }
 
