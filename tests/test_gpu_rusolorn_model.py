@@ -222,6 +222,44 @@ def test_greedy_generation_through_the_entry_point(name, dtype, folders):
     llm.runner.cache.check_invariants()
 
 
+def test_command_line_writes_a_random_model_and_generates_from_it(tmp_path):
+    """The command line on a configuration file alone: seeded random weights into a folder, then greedy generation and
+    sampling with a temperature, top-k and top-p from that folder."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    config_file, folder, out_file = tmp_path / "config.json", tmp_path / "model", tmp_path / "out.jsonl"
+    config_file.write_text(json.dumps(RUSOLORN["D"]["config"].to_dict()))
+    cli = [sys.executable, "-m", "somi_inference_amd.entrypoints.cli"]
+    done = subprocess.run(cli + ["--write-random-model", str(folder), "--config-json", str(config_file), "--random-seed", "3"],
+                          cwd=root, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    prompt = token_ids(vocab_of("D"), 9, 4)
+    common = ["--model-name", str(folder), "--dtype", "float32", "--num-blocks", "8", "--max-new-tokens", "6",
+              "--prompt-ids", ",".join(map(str, prompt)), "--output-file", str(out_file)]
+    done = subprocess.run(cli + common + ["--temperature", "0.0"], cwd=root, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    record = json.loads(done.stdout.strip().splitlines()[-1])
+    config, weights = load_plain(str(folder))
+    sequence = list(prompt)
+    for token in record["output"]:
+        logits = plain.forward(config, weights, sequence)[-1]
+        assert float(logits.max() - logits[token]) < 1e-4
+        sequence.append(token)
+    assert record["prompt"] == prompt and len(record["output"]) == 6
+    done = subprocess.run(cli + common + ["--temperature", "0.9", "--top-k", "5", "--top-p", "0.9", "--seed", "7"],
+                          cwd=root, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    sampled = json.loads(done.stdout.strip().splitlines()[-1])["output"]
+    sequence = list(prompt)
+    for token in sampled:                      # every sampled token is among the five most likely ones
+        logits = plain.forward(config, weights, sequence)[-1]
+        assert token in logits.topk(5).indices.tolist()
+        sequence.append(token)
+
+
 def test_a_preempted_request_is_recomputed_from_an_empty_state(folders):
     """A pool too small for three requests: one is preempted, gives back its pages and its state slot, and is run
     again from its first token later; its recurrent state and its convolution's inputs must start from zero again."""
