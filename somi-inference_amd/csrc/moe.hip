@@ -25,47 +25,57 @@ __device__ __forceinline__ float clamped_glu(float g, float u, float limit, floa
 }
 
 // The router's logits for widths that are a multiple of 4: a workgroup owns ROUTE_TOKENS tokens and ROUTE_EXPERTS
-// experts (8 a wavefront); the tokens' x goes through LDS 256 channels at a time, a lane multiplies 4 channels of every
-// chunk, and a (token, expert) sum is the lanes' partial sums added by `wave_sum`: one order whatever else runs.
+// experts (2 a wavefront: few, so that a step of a few tokens still spreads over several workgroups); the tokens' x
+// goes through LDS ROUTE_CHUNK channels at a time, a lane multiplies 4 channels of every 256 of a chunk (its loads of a
+// chunk are all asked for before any is used), and a (token, expert) sum is the lanes' partial sums added by
+// `wave_sum`: one order whatever else runs.
 #define ROUTE_TOKENS 8
-#define ROUTE_EXPERTS 32
+#define ROUTE_EXPERTS 8
+#define ROUTE_CHUNK 1024
 typedef __attribute__((ext_vector_type(4))) float route_f32x4;
 
 template <typename T>
 __global__ void __launch_bounds__(256)
 moe_router_logits_kernel(const T* __restrict__ x, int64_t row_stride, const float* __restrict__ router, int n_tokens,
                          int width, int experts, float* __restrict__ logits /*[N, experts]*/) {
-    __shared__ __attribute__((aligned(16))) float xs[ROUTE_TOKENS][256];
+    __shared__ __attribute__((aligned(16))) float xs[ROUTE_TOKENS][ROUTE_CHUNK];
+    constexpr int EPW = ROUTE_EXPERTS / 4, PIECES = ROUTE_CHUNK / 256;
     const int t0 = blockIdx.x * ROUTE_TOKENS;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int e0 = blockIdx.y * ROUTE_EXPERTS + wave * (ROUTE_EXPERTS / 4);
-    float acc[ROUTE_EXPERTS / 4][ROUTE_TOKENS];
+    const int e0 = blockIdx.y * ROUTE_EXPERTS + wave * EPW;
+    float acc[EPW][ROUTE_TOKENS];
 #pragma unroll
-    for (int ei = 0; ei < ROUTE_EXPERTS / 4; ++ei)
+    for (int ei = 0; ei < EPW; ++ei)
 #pragma unroll
         for (int tt = 0; tt < ROUTE_TOKENS; ++tt) acc[ei][tt] = 0.f;
-    for (int k0 = 0; k0 < width; k0 += 256) {
+    for (int k0 = 0; k0 < width; k0 += ROUTE_CHUNK) {
         __syncthreads();
-        for (int i = threadIdx.x; i < ROUTE_TOKENS * 256; i += 256) {
-            const int tt = i >> 8, k = k0 + (i & 255);
-            xs[tt][i & 255] = (t0 + tt < n_tokens && k < width) ? to_float(x[(int64_t)(t0 + tt) * row_stride + k]) : 0.f;
+        for (int i = threadIdx.x; i < ROUTE_TOKENS * ROUTE_CHUNK; i += 256) {
+            const int tt = i / ROUTE_CHUNK, k = k0 + (i % ROUTE_CHUNK);
+            xs[tt][i % ROUTE_CHUNK] = (t0 + tt < n_tokens && k < width) ? to_float(x[(int64_t)(t0 + tt) * row_stride + k]) : 0.f;
         }
+        route_f32x4 w[EPW][PIECES];
+#pragma unroll
+        for (int ei = 0; ei < EPW; ++ei)
+#pragma unroll
+            for (int j = 0; j < PIECES; ++j) {
+                const int k = k0 + j * 256 + lane * 4;
+                w[ei][j] = route_f32x4{0.f, 0.f, 0.f, 0.f};
+                if (e0 + ei < experts && k < width) w[ei][j] = *reinterpret_cast<const route_f32x4*>(router + (int64_t)(e0 + ei) * width + k);
+            }
         __syncthreads();
-        const int k = k0 + lane * 4;
-        route_f32x4 xv[ROUTE_TOKENS];
 #pragma unroll
-        for (int tt = 0; tt < ROUTE_TOKENS; ++tt) xv[tt] = *reinterpret_cast<const route_f32x4*>(&xs[tt][lane * 4]);
+        for (int j = 0; j < PIECES; ++j)
 #pragma unroll
-        for (int ei = 0; ei < ROUTE_EXPERTS / 4; ++ei) {
-            route_f32x4 w = {0.f, 0.f, 0.f, 0.f};
-            if (e0 + ei < experts && k < width) w = *reinterpret_cast<const route_f32x4*>(router + (int64_t)(e0 + ei) * width + k);
+            for (int tt = 0; tt < ROUTE_TOKENS; ++tt) {
+                const route_f32x4 xv = *reinterpret_cast<const route_f32x4*>(&xs[tt][j * 256 + lane * 4]);
 #pragma unroll
-            for (int tt = 0; tt < ROUTE_TOKENS; ++tt)
-                acc[ei][tt] += w[0] * xv[tt][0] + w[1] * xv[tt][1] + w[2] * xv[tt][2] + w[3] * xv[tt][3];
-        }
+                for (int ei = 0; ei < EPW; ++ei)
+                    acc[ei][tt] += w[ei][j][0] * xv[0] + w[ei][j][1] * xv[1] + w[ei][j][2] * xv[2] + w[ei][j][3] * xv[3];
+            }
     }
 #pragma unroll
-    for (int ei = 0; ei < ROUTE_EXPERTS / 4; ++ei)
+    for (int ei = 0; ei < EPW; ++ei)
 #pragma unroll
         for (int tt = 0; tt < ROUTE_TOKENS; ++tt) {
             const float total = wave_sum(acc[ei][tt]);

@@ -120,7 +120,7 @@ def attention_part(width, heads, groups, dim, window, scale, eps=1e-5):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,groups,dim,window,page,tokens", [(4, 2, 16, 24, 16, 150), (3, 3, 24, 1000, 8, 70),
                                                                (6, 2, 48, 56, 16, 300), (2, 1, 20, 1, 4, 30),
-                                                               (2, 2, 64, 7, 8, 90)])
+                                                               (2, 2, 64, 7, 8, 90), (4, 1, 128, 100, 16, 300)])
 def test_tied_value_attention_against_the_plain_function(dtype, heads, groups, dim, window, page, tokens):
     width = 64
     part = attention_part(width, heads, groups, dim, window, 0.9 * dim ** -0.5)
