@@ -394,7 +394,10 @@ typedef __attribute__((ext_vector_type(4))) float moe_f32x4;
 #define MOE_MFMA_ROWS 64
 #define MOE_MFMA_FRAGS (MOE_MFMA_ROWS / 16)
 
-template <bool GATED>
+// FRAGS: row fragments of a tile (4: up to 64 rows; 1: up to 16 rows, for steps of a few tokens, where a tile is an
+// expert's one or two rows and the time is the weights' way from memory).  KS: K steps of 32 whose fragments are asked
+// for together, a round ahead (1 with four row fragments; 4 with one, so that a lane has twenty loads in flight).
+template <bool GATED, int FRAGS, int KS>
 __global__ void __launch_bounds__(256)
 moe_product_mfma_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16* __restrict__ w,
                         const int* __restrict__ tiles, const int* __restrict__ order,
@@ -410,10 +413,10 @@ moe_product_mfma_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16
     if (col0 >= n_out) return;
     const bf16* wg = w + (int64_t)expert * (GATED ? 2 : 1) * n_out * K;
     // this lane's rows of the two operands
-    const bf16* arow[MOE_MFMA_FRAGS];
-    bool alive[MOE_MFMA_FRAGS];
+    const bf16* arow[FRAGS];
+    bool alive[FRAGS];
 #pragma unroll
-    for (int f = 0; f < MOE_MFMA_FRAGS; ++f) {
+    for (int f = 0; f < FRAGS; ++f) {
         const int row = f * 16 + r;
         alive[f] = row < rows;
         const int64_t src = alive[f] ? (GATED ? (int64_t)(order[first + row] / top) : (int64_t)(first + row)) : 0;
@@ -430,40 +433,48 @@ moe_product_mfma_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16
         brow[c] = wg + (blive[c] ? wrow : 0) * K + g * 8;
     }
     const int frags = (rows + 15) >> 4;               // the same for the whole workgroup
-    moe_f32x4 acc[MOE_MFMA_FRAGS][4];
+    moe_f32x4 acc[FRAGS][4];
 #pragma unroll
-    for (int f = 0; f < MOE_MFMA_FRAGS; ++f)
+    for (int f = 0; f < FRAGS; ++f)
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[f][c] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
     const moe_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    moe_bf16x8 fa[MOE_MFMA_FRAGS], fb[4], na[MOE_MFMA_FRAGS], nb[4];
-    auto fetch = [&](moe_bf16x8 (&xa)[MOE_MFMA_FRAGS], moe_bf16x8 (&xb)[4], int k0) {
-        const bool inside = k0 + g * 8 < K;
+    moe_bf16x8 fa[KS][FRAGS], fb[KS][4], na[KS][FRAGS], nb[KS][4];
+    auto fetch = [&](moe_bf16x8 (&xa)[KS][FRAGS], moe_bf16x8 (&xb)[KS][4], int k0) {
 #pragma unroll
-        for (int f = 0; f < MOE_MFMA_FRAGS; ++f)
-            xa[f] = (inside && alive[f]) ? *reinterpret_cast<const moe_bf16x8*>(arow[f] + k0) : zero;
+        for (int s = 0; s < KS; ++s) {
+            const bool inside = k0 + s * 32 + g * 8 < K;
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
-            xb[c] = (inside && blive[c]) ? *reinterpret_cast<const moe_bf16x8*>(brow[c] + k0) : zero;
+            for (int f = 0; f < FRAGS; ++f)
+                xa[s][f] = (inside && alive[f]) ? *reinterpret_cast<const moe_bf16x8*>(arow[f] + k0 + s * 32) : zero;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                xb[s][c] = (inside && blive[c]) ? *reinterpret_cast<const moe_bf16x8*>(brow[c] + k0 + s * 32) : zero;
+        }
     };
     fetch(fa, fb, 0);
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        if (k0 + 32 < K) fetch(na, nb, k0 + 32);
+    for (int k0 = 0; k0 < K; k0 += 32 * KS) {
+        if (k0 + 32 * KS < K) fetch(na, nb, k0 + 32 * KS);
 #pragma unroll
-        for (int f = 0; f < MOE_MFMA_FRAGS; ++f)
-            if (f < frags) {
+        for (int s = 0; s < KS; ++s)
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    acc[f][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[f], fb[c], acc[f][c], 0, 0, 0);
-            }
+            for (int f = 0; f < FRAGS; ++f)
+                if (f < frags) {
 #pragma unroll
-        for (int f = 0; f < MOE_MFMA_FRAGS; ++f) fa[f] = na[f];
+                    for (int c = 0; c < 4; ++c)
+                        acc[f][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s][f], fb[s][c], acc[f][c], 0, 0, 0);
+                }
 #pragma unroll
-        for (int c = 0; c < 4; ++c) fb[c] = nb[c];
+        for (int s = 0; s < KS; ++s) {
+#pragma unroll
+            for (int f = 0; f < FRAGS; ++f) fa[s][f] = na[s][f];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) fb[s][c] = nb[s][c];
+        }
     }
     // a lane holds rows g * 4 + i of a fragment's 16 and column r of its 16
 #pragma unroll
-    for (int f = 0; f < MOE_MFMA_FRAGS; ++f)
+    for (int f = 0; f < FRAGS; ++f)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int row = f * 16 + g * 4 + i;
@@ -613,8 +624,8 @@ extern "C" int somi_moe_product_mfma(const void* a, int64_t a_stride, const void
                                      int max_tiles, int tile_rows, const int* order, const float* pair_weight, int top,
                                      int n_out, int K, float limit, float alpha, float shift, void* out,
                                      hipStream_t stream) {
-    SOMI_REQUIRE(tile_rows == MOE_MFMA_ROWS || tile_rows == MOE_BIG_ROWS, "moe_product_mfma: tiles of %d rows (%d or %d)",
-                 tile_rows, MOE_MFMA_ROWS, MOE_BIG_ROWS);
+    SOMI_REQUIRE(tile_rows == 16 || tile_rows == MOE_MFMA_ROWS || tile_rows == MOE_BIG_ROWS,
+                 "moe_product_mfma: tiles of %d rows (16, %d or %d)", tile_rows, MOE_MFMA_ROWS, MOE_BIG_ROWS);
     SOMI_REQUIRE(max_tiles >= 0 && n_out > 0 && K > 0 && top > 0 && a_stride >= K, "moe_product_mfma: bad sizes");
     SOMI_REQUIRE(K % 8 == 0 && a_stride % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0,
                  "moe_product_mfma: K of %d or rows that are not aligned to 16 bytes", K);
@@ -628,12 +639,19 @@ extern "C" int somi_moe_product_mfma(const void* a, int64_t a_stride, const void
         else
             hipLaunchKernelGGL(moe_product_mfma_big_kernel<false>, grid, dim3(256), 0, stream, (const bf16*)a, a_stride,
                                (const bf16*)w, tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
+    } else if (tile_rows == 16) {
+        if (gated)
+            hipLaunchKernelGGL((moe_product_mfma_kernel<true, 1, 4>), grid, dim3(256), 0, stream, (const bf16*)a, a_stride,
+                               (const bf16*)w, tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
+        else
+            hipLaunchKernelGGL((moe_product_mfma_kernel<false, 1, 4>), grid, dim3(256), 0, stream, (const bf16*)a, a_stride,
+                               (const bf16*)w, tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
     } else if (gated)
-        hipLaunchKernelGGL(moe_product_mfma_kernel<true>, grid, dim3(256), 0, stream, (const bf16*)a, a_stride, (const bf16*)w,
-                           tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
+        hipLaunchKernelGGL((moe_product_mfma_kernel<true, MOE_MFMA_FRAGS, 1>), grid, dim3(256), 0, stream, (const bf16*)a, a_stride,
+                           (const bf16*)w, tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
     else
-        hipLaunchKernelGGL(moe_product_mfma_kernel<false>, grid, dim3(256), 0, stream, (const bf16*)a, a_stride, (const bf16*)w,
-                           tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
+        hipLaunchKernelGGL((moe_product_mfma_kernel<false, MOE_MFMA_FRAGS, 1>), grid, dim3(256), 0, stream, (const bf16*)a, a_stride,
+                           (const bf16*)w, tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
     SOMI_LAUNCH_CHECK("moe_product_mfma");
     return 0;
 }

@@ -1087,11 +1087,17 @@ MOE_MFMA_ROWS = 64           # ... of the matrix-core products
 MOE_BIG_ROWS = 128           # ... and of the matrix-core products that stage the rows through LDS (experts with many rows)
 
 
+MOE_FEW_ROWS = 16            # ... of the matrix-core products of steps of a few tokens (an expert's one or two rows)
+
+
 def moe_tile_rows(pairs: int, experts: int, mfma: bool) -> int:
     """Rows of a tile for a step of ``pairs`` (token, expert) pairs: the plain products' where the matrix-core ones do
-    not apply; the large tile once an expert has a tile's worth of rows on average."""
+    not apply; else the small tile while an expert has a few rows on average, the large one once it has a middle
+    tile's worth."""
     if not mfma:
         return MOE_TILE_ROWS
+    if pairs <= experts * MOE_FEW_ROWS // 2:
+        return MOE_FEW_ROWS
     return MOE_BIG_ROWS if pairs >= experts * MOE_MFMA_ROWS else MOE_MFMA_ROWS
 
 
@@ -1134,7 +1140,7 @@ def moe_align(chosen: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS
 
 
 def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, top: int,
-                limit: float, alpha: float, shift: float, tile_rows: int = MOE_TILE_ROWS) -> torch.Tensor:
+                limit: float, alpha: float, shift: float, tile_rows: int = MOE_TILE_ROWS, mfma: bool = False) -> torch.Tensor:
     """act[p] = glu(W_gate[e] x[t], W_up[e] x[t]) for the sorted pairs p = (t, e); gate_up: [experts, 2 F, K], gate rows
     first -> [pairs, F]."""
     _need(x, "rows")
@@ -1144,7 +1150,7 @@ def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, tiles: torch.Tensor, ord
         raise KernelError(f"moe_gate_up: matrices {tuple(gate_up.shape)} do not fit rows of {x.shape[1]}")
     pairs = order.numel()
     act = torch.empty((pairs, two_f // 2), dtype=x.dtype, device=x.device)
-    if tile_rows != MOE_TILE_ROWS:
+    if mfma:
         _check(library().somi_moe_product_mfma(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(gate_up), 1, _ptr(tiles), tiles.shape[0],
                                                int(tile_rows), _ptr(order), None, int(top), two_f // 2, k, ctypes.c_float(limit),
                                                ctypes.c_float(alpha), ctypes.c_float(shift), _ptr(act), _stream()))
@@ -1156,7 +1162,7 @@ def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, tiles: torch.Tensor, ord
 
 
 def moe_down(act: torch.Tensor, down: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, weight: torch.Tensor,
-             top: int, tile_rows: int = MOE_TILE_ROWS) -> torch.Tensor:
+             top: int, tile_rows: int = MOE_TILE_ROWS, mfma: bool = False) -> torch.Tensor:
     """y[pair] = weight[pair] * W_down[e] act[p] -> [pairs, width] float32, at the pairs' own places."""
     _need(act, "activations")
     _need(down, "down matrices", act.dtype)
@@ -1165,7 +1171,7 @@ def moe_down(act: torch.Tensor, down: torch.Tensor, tiles: torch.Tensor, order: 
         raise KernelError(f"moe_down: matrices {tuple(down.shape)} do not fit activations of {act.shape[1]}")
     _need(weight, "pair weights", torch.float32)
     y = torch.empty((order.numel(), width), dtype=torch.float32, device=act.device)
-    if tile_rows != MOE_TILE_ROWS:
+    if mfma:
         _check(library().somi_moe_product_mfma(_ptr(act), ctypes.c_int64(act.stride(0)), _ptr(down), 0, _ptr(tiles), tiles.shape[0],
                                                int(tile_rows), _ptr(order), _ptr(weight), int(top), width, k, ctypes.c_float(0.0),
                                                ctypes.c_float(0.0), ctypes.c_float(0.0), _ptr(y), _stream()))

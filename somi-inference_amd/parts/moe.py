@@ -106,13 +106,14 @@ class RoutedExperts(FeedForward):
         with stage("router"):
             chosen, weight = ops.moe_route(x, self.router, self.top, self.groups, self.keep_groups)
             # bfloat16: the products run on the matrix cores, in tiles sized by the rows an expert gets in this step
-            rows = ops.moe_tile_rows(chosen.numel(), self.num_experts, ops.moe_mfma_supported(x, self.gate_up, self.down))
+            mfma = ops.moe_mfma_supported(x, self.gate_up, self.down)
+            rows = ops.moe_tile_rows(chosen.numel(), self.num_experts, mfma)
             order, _, tiles = ops.moe_align(chosen, self.num_experts, rows)
         with stage("experts gate_up"):
             act = ops.moe_gate_up(x, self.gate_up, tiles, order, self.top, self.unit.limit, self.unit.alpha, self.unit.shift,
-                                  tile_rows=rows)
+                                  tile_rows=rows, mfma=mfma)
         with stage("experts down"):
-            pairs = ops.moe_down(act, self.down, tiles, order, weight, self.top, tile_rows=rows)
+            pairs = ops.moe_down(act, self.down, tiles, order, weight, self.top, tile_rows=rows, mfma=mfma)
         shared = None
         if self.shared_size:
             unit = self.shared_unit
