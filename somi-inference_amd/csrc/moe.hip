@@ -34,7 +34,12 @@ __device__ __forceinline__ float clamped_glu(float g, float u, float limit, floa
 #define ROUTE_CHUNK 1024
 typedef __attribute__((ext_vector_type(4))) float route_f32x4;
 
-template <typename T>
+template <typename T> struct RouteVec;
+template <> struct RouteVec<float> { typedef __attribute__((ext_vector_type(4))) float type; static constexpr int N = 4; };
+template <> struct RouteVec<bf16> { typedef __attribute__((ext_vector_type(8))) __bf16 type; static constexpr int N = 8; };
+
+// WIDE: the rows of x are read 16 bytes at a time (rows aligned to 16 bytes, a width that is a multiple of the piece).
+template <typename T, bool WIDE>
 __global__ void __launch_bounds__(256)
 moe_router_logits_kernel(const T* __restrict__ x, int64_t row_stride, const float* __restrict__ router, int n_tokens,
                          int width, int experts, float* __restrict__ logits /*[N, experts]*/) {
@@ -50,9 +55,27 @@ moe_router_logits_kernel(const T* __restrict__ x, int64_t row_stride, const floa
         for (int tt = 0; tt < ROUTE_TOKENS; ++tt) acc[ei][tt] = 0.f;
     for (int k0 = 0; k0 < width; k0 += ROUTE_CHUNK) {
         __syncthreads();
-        for (int i = threadIdx.x; i < ROUTE_TOKENS * ROUTE_CHUNK; i += 256) {
-            const int tt = i / ROUTE_CHUNK, k = k0 + (i % ROUTE_CHUNK);
-            xs[tt][i % ROUTE_CHUNK] = (t0 + tt < n_tokens && k < width) ? to_float(x[(int64_t)(t0 + tt) * row_stride + k]) : 0.f;
+        if (WIDE) {
+            constexpr int VN = RouteVec<T>::N, LOADS = ROUTE_TOKENS * ROUTE_CHUNK / VN / 256;
+            typename RouteVec<T>::type piece[LOADS];
+#pragma unroll
+            for (int j = 0; j < LOADS; ++j) {
+                const int i = (threadIdx.x + 256 * j) * VN, tt = i / ROUTE_CHUNK, k = k0 + (i % ROUTE_CHUNK);
+                const bool in = t0 + tt < n_tokens && k < width;
+                piece[j] = *reinterpret_cast<const typename RouteVec<T>::type*>(x + (int64_t)(in ? t0 + tt : 0) * row_stride + (in ? k : 0));
+            }
+#pragma unroll
+            for (int j = 0; j < LOADS; ++j) {
+                const int i = (threadIdx.x + 256 * j) * VN, tt = i / ROUTE_CHUNK, k = k0 + (i % ROUTE_CHUNK);
+                const bool in = t0 + tt < n_tokens && k < width;
+#pragma unroll
+                for (int v = 0; v < VN; ++v) xs[tt][(i % ROUTE_CHUNK) + v] = in ? (float)piece[j][v] : 0.f;
+            }
+        } else {
+            for (int i = threadIdx.x; i < ROUTE_TOKENS * ROUTE_CHUNK; i += 256) {
+                const int tt = i / ROUTE_CHUNK, k = k0 + (i % ROUTE_CHUNK);
+                xs[tt][i % ROUTE_CHUNK] = (t0 + tt < n_tokens && k < width) ? to_float(x[(int64_t)(t0 + tt) * row_stride + k]) : 0.f;
+            }
         }
         route_f32x4 w[EPW][PIECES];
 #pragma unroll
@@ -230,12 +253,17 @@ extern "C" int somi_moe_route(const void* x, int dtype, int64_t row_stride, cons
     const bool tiled = logits != nullptr && width % 4 == 0 && (uintptr_t)router % 16 == 0;
     if (tiled) {
         const dim3 grid(ceil_div(n_tokens, ROUTE_TOKENS), ceil_div(experts, ROUTE_EXPERTS));
-        if (dtype == SOMI_F32)
-            hipLaunchKernelGGL(moe_router_logits_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, row_stride, router,
-                               n_tokens, width, experts, logits);
-        else
-            hipLaunchKernelGGL(moe_router_logits_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)x, row_stride, router,
-                               n_tokens, width, experts, logits);
+        const int piece = dtype == SOMI_F32 ? 4 : 8;
+        const bool wide = width % piece == 0 && row_stride % piece == 0 && (uintptr_t)x % 16 == 0;
+#define SOMI_ROUTE(T, W)                                                                                                  \
+    hipLaunchKernelGGL((moe_router_logits_kernel<T, W>), grid, dim3(256), 0, stream, (const T*)x, row_stride, router, n_tokens, \
+                       width, experts, logits)
+        if (dtype == SOMI_F32) {
+            if (wide) SOMI_ROUTE(float, true); else SOMI_ROUTE(float, false);
+        } else {
+            if (wide) SOMI_ROUTE(bf16, true); else SOMI_ROUTE(bf16, false);
+        }
+#undef SOMI_ROUTE
     }
     if (dtype == SOMI_F32)
         hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n_tokens), dim3(64), 0, stream, (const float*)x, row_stride, router,
@@ -662,23 +690,25 @@ __global__ void __launch_bounds__(256)
 moe_combine_kernel(const float* __restrict__ y, const T* __restrict__ shared_rows, int top, int width,
                    float* __restrict__ out) {
     const int64_t t = blockIdx.x;
-    for (int c = threadIdx.x; c < width; c += 256) {
-        float acc = 0.f;
-        for (int j = 0; j < top; ++j) acc += y[(t * top + j) * width + c];
-        if (shared_rows != nullptr) acc += to_float(shared_rows[t * width + c]);
-        out[t * width + c] = acc;
-    }
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= width) return;
+    float acc = 0.f;
+    for (int j = 0; j < top; ++j) acc += y[(t * top + j) * width + c];
+    if (shared_rows != nullptr) acc += to_float(shared_rows[t * width + c]);
+    out[t * width + c] = acc;
 }
 
 extern "C" int somi_moe_combine(const float* y, const void* shared_rows, int shared_dtype, int n_tokens, int top, int width,
                                 float* out, hipStream_t stream) {
     SOMI_REQUIRE(n_tokens >= 0 && top > 0 && width > 0, "moe_combine: bad sizes");
     if (n_tokens == 0) return 0;
+    const dim3 grid(n_tokens, ceil_div(width, 256));
+    SOMI_REQUIRE(grid.y <= 65535, "moe_combine: rows too wide");
     if (shared_rows == nullptr || shared_dtype == SOMI_F32)
-        hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, y, (const float*)shared_rows, top,
+        hipLaunchKernelGGL(moe_combine_kernel<float>, grid, dim3(256), 0, stream, y, (const float*)shared_rows, top,
                            width, out);
     else if (shared_dtype == SOMI_BF16)
-        hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3(n_tokens), dim3(256), 0, stream, y, (const bf16*)shared_rows, top,
+        hipLaunchKernelGGL(moe_combine_kernel<bf16>, grid, dim3(256), 0, stream, y, (const bf16*)shared_rows, top,
                            width, out);
     else
         return somi_fail("moe_combine: unknown dtype %d", shared_dtype);
