@@ -527,125 +527,126 @@ moe_product_mfma_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16
         }
 }
 
-// The same for experts with many rows (prompt portions): a row tile of up to 128 sorted rows x 256 columns.  The rows'
-// part of a round of four K steps (128 rows x 128 values) goes through LDS, loaded once by the workgroup (rows padded by 16
-// bytes against bank conflicts), two buffers, one barrier a round; every wavefront reads all eight row fragments from LDS
-// and its own four column fragments of the weights straight from memory, a round (128 matrix instructions) ahead.  A weight fragment now serves eight row fragments instead of four, and the rows are read from memory once
-// instead of once a wavefront.
 #define MOE_BIG_ROWS 128
-#define MOE_BIG_FRAGS (MOE_BIG_ROWS / 16)
-#define MOE_BIG_KS 4                                        // K steps of 32 that one round of loads brings
-#define MOE_BIG_ROW_BYTES (MOE_BIG_KS * 64 + 16)            // a row's part of a round in LDS, padded against bank conflicts
-#define MOE_BIG_PIECES (MOE_BIG_ROWS * MOE_BIG_KS * 4 / 256) // 16-byte pieces of the rows a thread stages a round
+
+// The same for experts with many rows (prompt portions), both operands through LDS, `32x32x16` matrix instructions:
+// a workgroup owns a row tile of up to 128 sorted rows and 128 rows of the expert's matrix (GATED: 64 gate rows and the 64 up rows of the same columns), its four wavefronts a
+// 64 x 64 quarter each (two row fragments x two column fragments of 32; GATED: a wavefront's column fragments are gate
+// and up of the same 32 columns, so the gated unit needs no exchange).  A round is 64 values of K: every thread brings
+// four 16-byte pieces of the rows and four of the matrix into registers a round ahead and stores them into the LDS
+// buffer of the round (rows padded by 16 bytes: a fragment's 16-byte reads of 16 rows fall on different banks).
+typedef __attribute__((ext_vector_type(16))) float moe_f32x16;
+#define MOE_TILE_BK 64
+#define MOE_TILE_ROW_BYTES (MOE_TILE_BK * 2 + 16)
 
 template <bool GATED>
 __global__ void __launch_bounds__(256)
-moe_product_mfma_big_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16* __restrict__ w,
-                            const int* __restrict__ tiles, const int* __restrict__ order,
-                            const float* __restrict__ pair_weight, int top, int n_out, int K, float limit, float alpha,
-                            float shift, void* __restrict__ out_) {
-    __shared__ __attribute__((aligned(16))) char rows_lds[2][MOE_BIG_ROWS * MOE_BIG_ROW_BYTES];
+moe_product_tile_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16* __restrict__ w,
+                        const int* __restrict__ tiles, const int* __restrict__ order,
+                        const float* __restrict__ pair_weight, int top, int n_out, int K, float limit, float alpha,
+                        float shift, void* __restrict__ out_) {
+    __shared__ __attribute__((aligned(16))) char lds_a[2][128 * MOE_TILE_ROW_BYTES];
+    __shared__ __attribute__((aligned(16))) char lds_b[2][128 * MOE_TILE_ROW_BYTES];
     const int expert = tiles[blockIdx.x * 3];
     if (expert < 0) return;
     const int first = tiles[blockIdx.x * 3 + 1], rows = tiles[blockIdx.x * 3 + 2];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int r = lane & 15, g = lane >> 4;
-    constexpr int WAVE_COLS = GATED ? 32 : 64;
-    constexpr int ROUND = MOE_BIG_KS * 32;                      // K values of a round
-    constexpr int PPR = MOE_BIG_KS * 4;                         // 16-byte pieces of a row in a round
-    const int col0 = (blockIdx.y * 4 + wave) * WAVE_COLS;      // may lie past n_out: the wavefront then only helps to stage
+    const int wm = wave >> 1, wn = wave & 1;
+    const int frow = lane & 31, fk = lane >> 5;
+    constexpr int COLS = GATED ? 64 : 128;                      // output columns of a workgroup
+    const int col_base = blockIdx.y * COLS;
     const bf16* wg = w + (int64_t)expert * (GATED ? 2 : 1) * n_out * K;
-    // the pieces of the rows' round that this thread stages: piece p = tid + 256 j is piece p % PPR of row p / PPR
-    const bf16* srow[MOE_BIG_PIECES];
-    int sk[MOE_BIG_PIECES], slds[MOE_BIG_PIECES];
-#pragma unroll
-    for (int j = 0; j < MOE_BIG_PIECES; ++j) {
-        const int p = tid + 256 * j, row = p / PPR, piece = p % PPR;
-        const bool live = row < rows;
-        const int64_t src = live ? (GATED ? (int64_t)(order[first + row] / top) : (int64_t)(first + row)) : 0;
-        srow[j] = a + src * a_stride + piece * 8;
-        sk[j] = live ? piece * 8 : K;                            // a dead row's pieces count as past K: zeros
-        slds[j] = row * MOE_BIG_ROW_BYTES + piece * 16;
-    }
+    // the pieces a thread stages: piece p = tid + 256 j is the 16 bytes p % 8 of row p / 8 (of the rows and of the matrix)
+    const bf16* arow[4];
     const bf16* brow[4];
-    bool blive[4];
+    bool alive[4], blive[4];
+    int soff[4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const int col = GATED ? col0 + (c & 1) * 16 + r : col0 + c * 16 + r;
-        blive[c] = col < n_out;
-        const int64_t wrow = GATED ? (int64_t)(c >> 1) * n_out + col : (int64_t)col;
-        brow[c] = wg + (blive[c] ? wrow : 0) * K + g * 8;
+    for (int j = 0; j < 4; ++j) {
+        const int p = tid + 256 * j, row = p >> 3, piece = p & 7;
+        soff[j] = row * MOE_TILE_ROW_BYTES + piece * 16;
+        alive[j] = row < rows;
+        const int64_t src = alive[j] ? (GATED ? (int64_t)(order[first + row] / top) : (int64_t)(first + row)) : 0;
+        arow[j] = a + src * a_stride + piece * 8;
+        // LDS row of the matrix: wavefront column wn' = row / 64, its fragment f = (row / 32) % 2, column c = row % 32
+        const int wq = row >> 6, f = (row >> 5) & 1, c = row & 31;
+        const int col = GATED ? col_base + wq * 32 + c : col_base + wq * 64 + f * 32 + c;
+        blive[j] = col < n_out;
+        const int64_t wrow = GATED ? (int64_t)f * n_out + col : (int64_t)col;
+        brow[j] = wg + (blive[j] ? wrow : 0) * K + piece * 8;
     }
-    const int frags = (rows + 15) >> 4;
-    moe_f32x4 acc[MOE_BIG_FRAGS][4];
+    const int mfrags = min(2, (rows - wm * 64 + 31) >> 5);     // row fragments of this wavefront that hold rows (<= 0: none)
+    moe_f32x16 acc[2][2];
 #pragma unroll
-    for (int f = 0; f < MOE_BIG_FRAGS; ++f)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc[f][c] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     const moe_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    moe_bf16x8 sa[MOE_BIG_PIECES], fb[MOE_BIG_KS][4], nb[MOE_BIG_KS][4];
-    auto fetch = [&](moe_bf16x8 (&xa)[MOE_BIG_PIECES], moe_bf16x8 (&xb)[MOE_BIG_KS][4], int k0) {
+    moe_bf16x8 sa[4], sb[4];
+    auto fetch = [&](int k0) {
 #pragma unroll
-        for (int j = 0; j < MOE_BIG_PIECES; ++j)
-            xa[j] = k0 + sk[j] < K ? *reinterpret_cast<const moe_bf16x8*>(srow[j] + k0) : zero;
-#pragma unroll
-        for (int s = 0; s < MOE_BIG_KS; ++s) {
-            const bool inside = k0 + s * 32 + g * 8 < K;
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                xb[s][c] = (inside && blive[c]) ? *reinterpret_cast<const moe_bf16x8*>(brow[c] + k0 + s * 32) : zero;
+        for (int j = 0; j < 4; ++j) {
+            const bool inside = k0 + ((tid + 256 * j) & 7) * 8 < K;
+            sa[j] = (inside && alive[j]) ? *reinterpret_cast<const moe_bf16x8*>(arow[j] + k0) : zero;
+            sb[j] = (inside && blive[j]) ? *reinterpret_cast<const moe_bf16x8*>(brow[j] + k0) : zero;
         }
     };
-    fetch(sa, fb, 0);
+    fetch(0);
     int buf = 0;
-    for (int k0 = 0; k0 < K; k0 += ROUND, buf ^= 1) {
+    for (int k0 = 0; k0 < K; k0 += MOE_TILE_BK, buf ^= 1) {
 #pragma unroll
-        for (int j = 0; j < MOE_BIG_PIECES; ++j) *reinterpret_cast<moe_bf16x8*>(rows_lds[buf] + slds[j]) = sa[j];
-        __syncthreads();
-        if (k0 + ROUND < K) fetch(sa, nb, k0 + ROUND);
-#pragma unroll
-        for (int s = 0; s < MOE_BIG_KS; ++s) {
-            if (k0 + s * 32 >= K) break;
-#pragma unroll
-            for (int f = 0; f < MOE_BIG_FRAGS; ++f)
-                if (f < frags) {
-                    const moe_bf16x8 fa = *reinterpret_cast<const moe_bf16x8*>(
-                        rows_lds[buf] + (f * 16 + r) * MOE_BIG_ROW_BYTES + s * 64 + g * 16);
-#pragma unroll
-                    for (int c = 0; c < 4; ++c)
-                        acc[f][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, fb[s][c], acc[f][c], 0, 0, 0);
-                }
+        for (int j = 0; j < 4; ++j) {
+            *reinterpret_cast<moe_bf16x8*>(lds_a[buf] + soff[j]) = sa[j];
+            *reinterpret_cast<moe_bf16x8*>(lds_b[buf] + soff[j]) = sb[j];
         }
+        __syncthreads();
+        if (k0 + MOE_TILE_BK < K) fetch(k0 + MOE_TILE_BK);
+        if (mfrags > 0) {
 #pragma unroll
-        for (int s = 0; s < MOE_BIG_KS; ++s)
+            for (int ks = 0; ks < MOE_TILE_BK / 16; ++ks) {
+                moe_bf16x8 fa[2], fb[2];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) fb[s][c] = nb[s][c];
-    }
-    if (col0 >= n_out) return;
+                for (int i = 0; i < 2; ++i)
+                    fa[i] = *reinterpret_cast<const moe_bf16x8*>(lds_a[buf] + (wm * 64 + i * 32 + frow) * MOE_TILE_ROW_BYTES + ks * 32 + fk * 16);
 #pragma unroll
-    for (int f = 0; f < MOE_BIG_FRAGS; ++f)
+                for (int j = 0; j < 2; ++j)
+                    fb[j] = *reinterpret_cast<const moe_bf16x8*>(lds_b[buf] + (wn * 64 + j * 32 + frow) * MOE_TILE_ROW_BYTES + ks * 32 + fk * 16);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int row = f * 16 + g * 4 + i;
-            if (row >= rows) continue;
-            if (GATED) {
+                for (int i = 0; i < 2; ++i)
+                    if (i < mfrags) {
 #pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    const int col = col0 + c * 16 + r;
-                    if (col < n_out)
-                        ((bf16*)out_)[(int64_t)(first + row) * n_out + col] =
-                            (bf16)clamped_glu(acc[f][c][i], acc[f][c + 2][i], limit, alpha, shift);
-                }
-            } else {
-                const int pair = order[first + row];
-                const float pw = pair_weight[pair];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const int col = col0 + c * 16 + r;
-                    if (col < n_out) ((float*)out_)[(int64_t)pair * n_out + col] = pw * acc[f][c][i];
-                }
+                        for (int j = 0; j < 2; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);   // D[row][column]
+                    }
             }
         }
+    }
+    // D[row][column]: lane l has column l % 32 of a fragment and, in registers 4 g .. 4 g + 3, the rows 8 g + 4 (l / 32) + 0..3
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = wm * 64 + i * 32 + 8 * g + 4 * fk + e;
+                if (row >= rows) continue;
+                if (GATED) {
+                    const int col = col_base + wn * 32 + frow;
+                    if (col < n_out)
+                        ((bf16*)out_)[(int64_t)(first + row) * n_out + col] =
+                            (bf16)clamped_glu(acc[i][0][4 * g + e], acc[i][1][4 * g + e], limit, alpha, shift);
+                } else {
+                    const int pair = order[first + row];
+                    const float pw = pair_weight[pair];
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const int col = col_base + wn * 64 + j * 32 + frow;
+                        if (col < n_out) ((float*)out_)[(int64_t)pair * n_out + col] = pw * acc[i][j][4 * g + e];
+                    }
+                }
+            }
 }
 
 extern "C" int somi_moe_product_mfma(const void* a, int64_t a_stride, const void* w, int gated, const int* tiles,
@@ -661,11 +662,13 @@ extern "C" int somi_moe_product_mfma(const void* a, int64_t a_stride, const void
     const dim3 grid(max_tiles, ceil_div(n_out, gated ? 128 : 256));
     SOMI_REQUIRE(grid.y <= 65535, "moe_product_mfma: too many columns");
     if (tile_rows == MOE_BIG_ROWS) {
+        const dim3 tgrid(max_tiles, ceil_div(n_out, gated ? 64 : 128));
+        SOMI_REQUIRE(tgrid.y <= 65535, "moe_product_mfma: too many columns");
         if (gated)
-            hipLaunchKernelGGL(moe_product_mfma_big_kernel<true>, grid, dim3(256), 0, stream, (const bf16*)a, a_stride,
+            hipLaunchKernelGGL(moe_product_tile_kernel<true>, tgrid, dim3(256), 0, stream, (const bf16*)a, a_stride,
                                (const bf16*)w, tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
         else
-            hipLaunchKernelGGL(moe_product_mfma_big_kernel<false>, grid, dim3(256), 0, stream, (const bf16*)a, a_stride,
+            hipLaunchKernelGGL(moe_product_tile_kernel<false>, tgrid, dim3(256), 0, stream, (const bf16*)a, a_stride,
                                (const bf16*)w, tiles, order, pair_weight, top, n_out, K, limit, alpha, shift, out);
     } else if (tile_rows == 16) {
         if (gated)
