@@ -533,8 +533,8 @@ moe_product_mfma_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16
 // a workgroup owns a row tile of up to 128 sorted rows and 128 rows of the expert's matrix (GATED: 64 gate rows and the 64 up rows of the same columns), its four wavefronts a
 // 64 x 64 quarter each (two row fragments x two column fragments of 32; GATED: a wavefront's column fragments are gate
 // and up of the same 32 columns, so the gated unit needs no exchange).  A round is 64 values of K: every thread brings
-// four 16-byte pieces of the rows and four of the matrix into registers a round ahead and stores them into the LDS
-// buffer of the round (rows padded by 16 bytes: a fragment's 16-byte reads of 16 rows fall on different banks).
+// four 16-byte pieces of the rows and four of the matrix into registers two rounds ahead (two sets of registers) and
+// stores them into the LDS buffer of the round (rows padded by 16 bytes: a fragment's 16-byte reads of 16 rows fall on different banks).
 typedef __attribute__((ext_vector_type(16))) float moe_f32x16;
 #define MOE_TILE_BK 64
 #define MOE_TILE_ROW_BYTES (MOE_TILE_BK * 2 + 16)
@@ -584,8 +584,9 @@ moe_product_tile_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     const moe_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    moe_bf16x8 sa[4], sb[4];
-    auto fetch = [&](int k0) {
+    // two sets of staging registers: a round's pieces are asked of memory two rounds before they go into LDS
+    moe_bf16x8 sa0[4], sb0[4], sa1[4], sb1[4];
+    auto fetch = [&](moe_bf16x8 (&sa)[4], moe_bf16x8 (&sb)[4], int k0) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const bool inside = k0 + ((tid + 256 * j) & 7) * 8 < K;
@@ -593,16 +594,14 @@ moe_product_tile_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16
             sb[j] = (inside && blive[j]) ? *reinterpret_cast<const moe_bf16x8*>(brow[j] + k0) : zero;
         }
     };
-    fetch(0);
-    int buf = 0;
-    for (int k0 = 0; k0 < K; k0 += MOE_TILE_BK, buf ^= 1) {
+    auto round = [&](moe_bf16x8 (&sa)[4], moe_bf16x8 (&sb)[4], int buf, int k_next) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             *reinterpret_cast<moe_bf16x8*>(lds_a[buf] + soff[j]) = sa[j];
             *reinterpret_cast<moe_bf16x8*>(lds_b[buf] + soff[j]) = sb[j];
         }
         __syncthreads();
-        if (k0 + MOE_TILE_BK < K) fetch(k0 + MOE_TILE_BK);
+        if (k_next < K) fetch(sa, sb, k_next);
         if (mfrags > 0) {
 #pragma unroll
             for (int ks = 0; ks < MOE_TILE_BK / 16; ++ks) {
@@ -622,6 +621,13 @@ moe_product_tile_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16
                     }
             }
         }
+    };
+    fetch(sa0, sb0, 0);
+    if (MOE_TILE_BK < K) fetch(sa1, sb1, MOE_TILE_BK);
+    for (int k0 = 0; k0 < K; k0 += 2 * MOE_TILE_BK) {
+        round(sa0, sb0, 0, k0 + 2 * MOE_TILE_BK);
+        if (k0 + MOE_TILE_BK >= K) break;
+        round(sa1, sb1, 1, k0 + 3 * MOE_TILE_BK);
     }
     // D[row][column]: lane l has column l % 32 of a fragment and, in registers 4 g .. 4 g + 3, the rows 8 g + 4 (l / 32) + 0..3
 #pragma unroll
