@@ -121,3 +121,26 @@ def test_kamedra_option_runs_both_models_and_leaves_the_default_alone():
         assert "attention" in line[model]["stages"]["prefill_512"]
     assert "recurrence" in line["kamedra"]["stages"]["prefill_512"] and line["value"] == line["kamedra"]["decode_b8"]["tok_s"]
     assert line["prefill_kernels"]["kamedra_attention"]["ms"] > 0 and line["decode_kernels"]["kamedra_recurrence"]["ms"] > 0
+
+
+def test_rusolorn_option_runs_both_models_and_leaves_the_default_alone():
+    """``--rusolorn`` runs a Rusolorn model beside the closest Kamedra model and prints one JSON line; the sizes' config
+    dictionaries build through the registry like any config.json."""
+    sys.path.insert(0, ROOT)
+    import bench
+    from somi_inference_amd.config import config_from_dict
+    for sizes in bench.RUSOLORN_SIZES:
+        arch, config = config_from_dict(bench.rusolorn_config_dict(sizes))
+        assert arch.name == "Rusolorn" and len(config.layers) == bench.RUSOLORN_LAYERS and config.layers[0].mlp.shared_ff
+        arch, closest = config_from_dict(bench.rusolorn_closest_config_dict(sizes))
+        assert arch.name == "Kamedra" and len(closest.layers) == bench.RUSOLORN_LAYERS
+        assert closest.layers[0].ff == config.layers[0].mlp.top * config.layers[0].mlp.ff + config.layers[0].mlp.shared_ff
+    done = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--rusolorn", "1b", "--steps", "16", "--warmup", "2",
+                           "--prefill-tokens", "512", "--context", "1024"], capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-3000:]
+    line = json.loads(done.stdout.strip().splitlines()[-1])
+    for model in ("rusolorn", "closest"):
+        assert line[model]["prefill"]["512"]["value"] > 0 and line[model]["decode_b8"]["tok_s"] > 0
+        assert "attention" in line[model]["stages"]["prefill_512"] and "recurrence" in line[model]["stages"]["prefill_512"]
+    assert "experts gate_up" in line["rusolorn"]["stages"]["prefill_512"] and line["value"] == line["rusolorn"]["decode_b8"]["tok_s"]
+    assert line["prefill_kernels"]["rusolorn_experts"]["ms"] > 0 and line["decode_kernels"]["rusolorn_recurrence"]["ms"] > 0
